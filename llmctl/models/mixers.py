@@ -13,11 +13,22 @@
   per-head temperature, chunked or windowed masks, a softmax sink.
 * :class:`CausalConv` — a short causal convolution over time per channel, its last inputs carried in a
   state slot; :class:`ClampedGLU` — a gated feed-forward with clamped branches.
+* :class:`GatedLinearAttention` — a matrix memory per head whose key rows decay by a data-dependent
+  factor per key channel (low-rank decay projection, temperature ``tau``), read out with the query,
+  RMS-normed per head and gated by ``silu``; its state lives in a slot pool like the mLSTM's.
+* :class:`SigmoidAttention` — grouped-query causal attention without softmax over the same paged row
+  cache ``[v | k]``: biases on q / k / v, RMS norm over the whole of q and of k, a query temperature that
+  grows with the logarithm of the position, a logarithmic distance penalty per head, key weights
+  ``sigmoid(score + head bias)`` that are not normalised, one sigmoid output gate per head.
+* :class:`DenseFF` — an ungated feed-forward ``W_down act(W_up h)``.
 * :class:`MLSTM` — the xLSTM matrix memory: per head a ``[dk, dv]`` state with exponential input gate,
   sigmoid forget gate (both soft-capped) and a running log-scale stabiliser; state lives in a slot
   pool of the engine's cache, one slot per live sequence.
 
-Both read a :class:`StepBatch` (the engine's description of one step: packed prompt portions first,
+The mixers take ``side`` extra output rows on their fused input projection (a layer's own gate or
+the like, which reads the same input) and hand those columns back beside their result.
+
+All read a :class:`StepBatch` (the engine's description of one step: packed prompt portions first,
 then one row per decoding sequence) and the layer's part of the engine's cache.  Projections are
 vendor GEMMs on fused weights; everything else is a kernel of :mod:`llmctl.ops.hybrid`.
 """
@@ -25,7 +36,7 @@ vendor GEMMs on fused weights; everything else is a kernel of :mod:`llmctl.ops.h
 from __future__ import annotations
 
 import math
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Optional
 
 import torch
@@ -57,6 +68,7 @@ class StepBatch:
     seq_of: Optional[torch.Tensor] = None  # int32 [T] index (into cu / start / state) of every row's sequence
     d_max_ctx: int = 0  # the longest context among the decoding sequences
     fresh: bool = False  # every row belongs to a prompt portion that starts at position 0 (no earlier context)
+    scratch: dict = field(default_factory=dict)  # what layers derive from the step alone and share (chunk plans of scans)
 
 
 def rotary_frequencies(base: float, dims: int, scaling: Optional[dict] = None, device=None):
@@ -335,3 +347,150 @@ class MLSTM(nn.Module):
         o = hops.mlstm_scan(q, k, v, gates, self.b_i, self.b_f, self.cap, 1.0 / math.sqrt(dk), S, n, m, b.state,
                             b.cu, b.start, cu_host=b.cu_host)
         return F.linear(hops.headnorm_gate(o, self.norm, g, self.eps, h.dtype), self.w_o)
+
+
+def _mm_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """``x @ w^T`` with an fp32 result (inputs in their own dtype, fp32 accumulation)."""
+    if x.dtype == torch.float32:
+        return F.linear(x, w)
+    try:
+        return torch.mm(x, w.t(), out_dtype=torch.float32)
+    except (TypeError, RuntimeError):
+        return F.linear(x, w).float()
+
+
+class GatedLinearAttention(nn.Module):
+    """Per head a memory ``S [dim, vdim]``: ``S_t = diag(a_t) S_(t-1) + k_t v_t^T``, ``o_t = S_t^T q_t`` with
+    ``q = W_q h * dim^-1/2`` and the decay ``a_t = sigmoid(W_a2 (W_a1 h) + b)^(1/tau)`` per key channel.
+    Each head's ``o`` is RMS-normed over vdim (one weight ``[vdim]`` for all heads), the heads are
+    concatenated, multiplied by ``silu(W_g h)`` and projected by ``W_o``.  The fused input weight is
+    ``[W_q ; W_k ; W_v ; W_g ; W_a1 ; side rows]``."""
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, tau: float, decay_rank: int, eps: float,
+                 side: int = 0, device=None, dtype=None):
+        super().__init__()
+        self.width, self.H, self.dk, self.dv, self.tau, self.rank, self.eps = width, heads, dim, vdim, float(tau), decay_rank, eps
+        self.side = side
+        kw = dict(device=device, dtype=dtype)
+        f32 = dict(device=device, dtype=torch.float32)
+        self.cols = 2 * heads * dim + 2 * heads * vdim + decay_rank
+        self.w_in = nn.Parameter(torch.empty(self.cols + side, width, **kw))
+        self.b_in = nn.Parameter(torch.zeros(self.cols + side, **kw)) if side else None  # only side rows carry a bias
+        self.w_a2 = nn.Parameter(torch.empty(heads * dim, decay_rank, **kw))
+        self.b_a2 = nn.Parameter(torch.zeros(heads * dim, **f32))
+        self.norm = nn.Parameter(torch.ones(vdim, **f32))
+        self.w_o = nn.Parameter(torch.empty(width, heads * vdim, **kw))
+        for w in (self.w_in, self.w_a2, self.w_o):
+            _init(w, 0.02)
+        self._nw = None
+
+    cache_kind = "state"
+    cache_row = 0
+
+    def state_shapes(self):
+        return [(self.H, self.dk, self.dv)]
+
+    def _norm_rows(self) -> torch.Tensor:
+        """The per-head norm weight repeated for every head (made once; serving weights are static)."""
+        key = (self.norm.data_ptr(), self.norm._version, self.norm.device)
+        if self._nw is None or self._nw[0] != key:
+            self._nw = (key, self.norm.detach().repeat(self.H).contiguous())
+        return self._nw[1]
+
+    def step(self, h: torch.Tensor, b: StepBatch, state):
+        if isinstance(state, tuple) and len(state) == 2 and isinstance(state[1], tuple):  # (rows, states)
+            state = state[1]
+        T, H, dk, dv = h.shape[0], self.H, self.dk, self.dv
+        z = F.linear(h, self.w_in, self.b_in)
+        a, c, e = H * dk, 2 * H * dk, 2 * H * dk + H * dv
+        q, k = z[:, :a].unflatten(1, (H, dk)), z[:, a:c].unflatten(1, (H, dk))
+        v = z[:, c:e].unflatten(1, (H, dv))
+        g = z[:, e:e + H * dv]
+        decay = _mm_f32(z[:, e + H * dv:self.cols], self.w_a2)  # fp32 [T, H * dk]
+        if "gla_plan" not in b.scratch:
+            b.scratch["gla_plan"] = hops.gla_chunk_plan(b.cu_host, h.device) if h.is_cuda else None
+        o = hops.gla_scan(q, k, v, decay, self.b_a2, self.tau, dk ** -0.5, state[0], b.state, b.cu, b.start,
+                          plan=b.scratch["gla_plan"])
+        y = F.linear(hops.headnorm_gate(o, self._norm_rows(), g, self.eps, h.dtype, silu=True), self.w_o)
+        return (y, z[:, self.cols:]) if self.side else y
+
+
+class SigmoidAttention(nn.Module):
+    """Grouped-query causal attention whose key weights are ``sigmoid(score + bias_h)``, not a softmax
+    (``heads`` query heads over ``kv_heads`` key / value heads; key size ``dim``, value size ``vdim``):
+    q, k, v with biases; RMS norm over all of q and all of k before the split into heads; no rotation;
+    ``q *= 1 + temp_coef ln(floor((p + 1) / temp_every) + 1)`` at position p; ``score = q . k * scale -
+    r1_h ln(1 + r2_h (i - j))``; head h's output times ``sigmoid(W_g h)_h``.  The cache row of a token is
+    ``[v | k]`` per kv head; the fused input weight is ``[W_q ; W_k ; W_v ; W_g ; side rows]``."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, eps: float,
+                 temp_coef: float = 0.0, temp_every: int = 1, window: Optional[int] = None, side: int = 0,
+                 device=None, dtype=None):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("kv heads must divide the heads")
+        self.width, self.H, self.G, self.dk, self.dv = width, heads, kv_heads, dim, vdim
+        self.scale, self.eps, self.temp_coef, self.temp_every = float(scale), eps, float(temp_coef), int(temp_every)
+        self.window = int(window) if window else hops.NO_LIMIT
+        self.side = side
+        kw = dict(device=device, dtype=dtype)
+        f32 = dict(device=device, dtype=torch.float32)
+        self.cols = (heads + kv_heads) * dim + kv_heads * vdim + heads
+        self.w_in = nn.Parameter(torch.empty(self.cols + side, width, **kw))
+        self.b_in = nn.Parameter(torch.zeros(self.cols + side, **kw))
+        self.q_norm = nn.Parameter(torch.ones(heads * dim, **f32))
+        self.k_norm = nn.Parameter(torch.ones(kv_heads * dim, **f32))
+        self.dist_a = nn.Parameter(torch.zeros(heads, **f32))  # r1
+        self.dist_b = nn.Parameter(torch.zeros(heads, **f32))  # r2
+        self.bias = nn.Parameter(torch.zeros(heads, **f32))
+        self.w_o = nn.Parameter(torch.empty(width, heads * vdim, **kw))
+        for w in (self.w_in, self.w_o):
+            _init(w, 0.02)
+
+    cache_kind = "latent"  # a paged pool of rows
+
+    @property
+    def cache_row(self) -> int:
+        return self.G * (self.dv + self.dk)
+
+    def state_shapes(self):
+        return []
+
+    def step(self, h: torch.Tensor, b: StepBatch, cache):
+        rows = cache[0] if isinstance(cache, tuple) else cache
+        T, H, G, dk, dv = h.shape[0], self.H, self.G, self.dk, self.dv
+        z = F.linear(h, self.w_in, self.b_in)
+        q = hops.qk_fullnorm_prep(z, H, G, dk, dv, self.q_norm, self.k_norm, self.eps, b.pos, self.temp_coef,
+                                  self.temp_every, rows, b.slots)
+        opt = dict(groups=G, koff=dv, sig_bias=self.bias, dist_a=self.dist_a, dist_b=self.dist_b)
+        outs = []
+        if b.Tp:
+            outs.append(hops.latent_attention_prefill(q[:b.Tp], rows, b.p_bt, b.p_cu, b.p_ctx, self.window, None,
+                                                      self.scale, dv, b.max_q, **opt))
+        if T > b.Tp:
+            outs.append(hops.latent_attention_decode(q[b.Tp:], rows, b.d_bt, b.d_ctx, self.window, None, self.scale, dv,
+                                                     max_ctx=b.d_max_ctx, **opt))
+        o = outs[0] if len(outs) == 1 else torch.cat(outs)
+        g0 = self.cols - H
+        y = F.linear(hops.sigmoid_gate_mul(o.reshape(T, H * dv), z[:, g0:self.cols]), self.w_o)
+        return (y, z[:, self.cols:]) if self.side else y
+
+
+class DenseFF(nn.Module):
+    """``W_down act(W_up h)`` with ``act`` one of :func:`llmctl.ops.hybrid.act_any`'s kinds; the up
+    projection carries ``side`` extra output rows (with a bias) that are handed back."""
+
+    def __init__(self, width: int, ff: int, act: str = "gelu", side: int = 0, device=None, dtype=None):
+        super().__init__()
+        self.ff, self.act, self.side = ff, act, side
+        kw = dict(device=device, dtype=dtype)
+        self.w_up = nn.Parameter(torch.empty(ff + side, width, **kw))
+        self.b_up = nn.Parameter(torch.zeros(ff + side, **kw)) if side else None
+        self.w_down = nn.Parameter(torch.empty(width, ff, **kw))
+        _init(self.w_up, 0.02)
+        _init(self.w_down, 0.02)
+
+    def forward(self, h: torch.Tensor):
+        z = F.linear(h, self.w_up, self.b_up)
+        y = F.linear(hops.act_any(z[:, :self.ff], self.act), self.w_down)
+        return (y, z[:, self.ff:]) if self.side else y

@@ -168,17 +168,27 @@ class MoEMLP(nn.Module):
         return dst, padded
 
 
-def run_expert_segments(xe: torch.Tensor, counts: List[int], ups, downs, act=None) -> torch.Tensor:
+def run_expert_segments(xe: torch.Tensor, counts: List[int], ups, downs, act=None, pad: int = 0) -> torch.Tensor:
     """``down_e(act(up_e(x)))`` on each expert's contiguous row segment of ``xe`` (rows sorted by
-    expert, ``counts[e]`` rows each)."""
+    expert, ``counts[e]`` rows each).
+
+    ``pad`` > 0: an expert's GEMMs also take the rows that follow its segment, up to the next multiple of
+    ``pad`` rows (of 16 for segments of at most 16 rows), and the results of those rows are dropped; ``xe``
+    must then hold ``pad`` spare rows after the last segment.  The GEMM library picks a kernel per shape and
+    remembers the pick: row counts that change with every step's routing cost ~60 us of host time per GEMM
+    for the lookup, a few recurring ones cost none."""
     act = act or ops.swiglu
     outs, o = [], 0
     for e, n in enumerate(counts):
         if n == 0:
             continue
-        seg = xe[o:o + n]
+        m = n
+        if pad:
+            m = 16 if n <= 16 else (n + pad - 1) // pad * pad
+            m = min(m, xe.shape[0] - o)
+        y = linear(act(linear(xe[o:o + m], ups[e])), downs[e])
+        outs.append(y[:n] if m != n else y)
         o += n
-        outs.append(linear(act(linear(seg, ups[e])), downs[e]))
     return torch.cat(outs, 0) if outs else xe.new_zeros((0, downs[0].shape[0]))
 
 
@@ -219,6 +229,85 @@ class GroupLimitedMoE(nn.Module):
         ye = run_expert_segments(x.index_select(0, tok), counts, self.experts_up, self.experts_down, hops.swiglu_any)
         w = topw.reshape(-1).index_select(0, order).unsqueeze(-1)
         return torch.zeros(T, x.shape[1], dtype=torch.float32, device=x.device).index_add_(0, tok, ye.float() * w)
+
+
+class BiasedSoftmaxMoE(nn.Module):
+    """Routed ungated experts ``W_down act(W_up h)`` chosen by softmax scores plus a selection bias
+    (serving forward).  Router logits are an fp32 product; ``s = softmax(z)``; the ``top`` experts with the
+    largest ``s + bias`` are used, weighted by their own ``s`` over the sum of the chosen ones; an
+    optional shared expert of the same form runs for every token.  Dispatch as in :class:`GroupLimitedMoE`
+    (token copies sorted by expert, per-expert GEMMs on contiguous segments, fp32 weighted sum).  Steps of
+    few tokens that between them reach about every expert anyway (decode batches) take the dense form
+    instead: all experts on all rows in one up GEMM, one activation pass and one batched down GEMM on the
+    stacked weights, the unchosen experts weighted by zero; that form has no host synchronisation and a
+    quarter of the launches.  The shared expert's up projection carries ``side`` extra output rows (with a
+    bias) that are handed back; without a shared expert they are a projection of their own."""
+
+    def __init__(self, width: int, ff: int, experts: int, top: int, act: str = "relu2", shared_ff: int = 0,
+                 side: int = 0, device=None, dtype=None):
+        super().__init__()
+        if not (0 < top <= experts):
+            raise ValueError("router: top must lie in 1 .. experts")
+        self.E, self.top, self.ff, self.act, self.shared_ff, self.side = experts, top, ff, act, shared_ff, side
+        kw = dict(device=device, dtype=dtype)
+        f32 = dict(device=device, dtype=torch.float32)
+        self.w_router = nn.Parameter(torch.empty(experts, width, **f32))
+        self.bias = nn.Parameter(torch.zeros(experts, **f32))
+        self.w_up = nn.Parameter(torch.empty(experts, ff, width, **kw))  # stacked: expert e is w_up[e]
+        self.w_down = nn.Parameter(torch.empty(experts, width, ff, **kw))
+        self.w_sup = nn.Parameter(torch.empty(shared_ff + side, width, **kw)) if shared_ff + side else None
+        self.b_sup = nn.Parameter(torch.zeros(shared_ff + side, **kw)) if side else None
+        self.w_sdown = nn.Parameter(torch.empty(width, shared_ff, **kw)) if shared_ff else None
+        with torch.no_grad():
+            self.w_router.normal_(0.0, 0.02)
+            for p in (self.w_up, self.w_down, self.w_sup, self.w_sdown):
+                if p is not None:
+                    p.normal_(0.0, 0.02)
+
+    @property
+    def experts_up(self):
+        return self.w_up.unbind(0)
+
+    @property
+    def experts_down(self):
+        return self.w_down.unbind(0)
+
+    PAD = 64  # expert segments run in multiples of this many rows
+    DENSE_ROWS = 64  # steps of at most this many rows may take the dense form
+
+    def _dense(self, T: int) -> bool:
+        return T <= self.DENSE_ROWS and T * self.top >= self.E
+
+    def forward(self, x: torch.Tensor):
+        """x [T, width] -> fp32 [T, width] (and the side columns)."""
+        from llmctl.ops import hybrid as hops
+
+        T = x.shape[0]
+        act = lambda u: hops.act_any(u, self.act)
+        topi, topw = hops.bias_topk_router(torch.nn.functional.linear(x.float(), self.w_router), self.bias, self.top)
+        if self._dense(T):
+            E, ff, W = self.E, self.ff, x.shape[1]
+            a = act(torch.nn.functional.linear(x, self.w_up.view(E * ff, W)))  # [T, E * ff]
+            y = torch.bmm(a.view(T, E, ff).transpose(0, 1), self.w_down.transpose(1, 2))  # [E, T, W]
+            dw = torch.zeros(T, E, dtype=torch.float32, device=x.device).scatter_(1, topi, topw)
+            out = (y.float() * dw.t().unsqueeze(-1)).sum(0)
+        else:
+            flat = topi.reshape(-1)
+            counts = torch.bincount(flat, minlength=self.E).tolist()  # the layer's one host sync
+            order = torch.argsort(flat, stable=True)
+            tok = torch.div(order, self.top, rounding_mode="floor")
+            xs = x.new_zeros((tok.shape[0] + self.PAD, x.shape[1]))  # spare rows: see run_expert_segments
+            torch.index_select(x, 0, tok, out=xs[:tok.shape[0]])
+            ye = run_expert_segments(xs, counts, self.experts_up, self.experts_down, act, pad=self.PAD)
+            w = topw.reshape(-1).index_select(0, order).unsqueeze(-1)
+            out = torch.zeros(T, x.shape[1], dtype=torch.float32, device=x.device).index_add_(0, tok, ye.float() * w)
+        side = None
+        if self.w_sup is not None:
+            z = torch.nn.functional.linear(x, self.w_sup, self.b_sup)
+            if self.shared_ff:
+                out += torch.nn.functional.linear(act(z[:, :self.shared_ff]), self.w_sdown)
+            side = z[:, self.shared_ff:]
+        return (out, side) if self.side else out
 
 
 def expert_param_global_name(name: str, module_e0: int) -> str:

@@ -54,5 +54,14 @@ def _register_builtin() -> None:
 
     register(dumalix.ARCHITECTURE, Family(dumalix.DumalixConfig, build_dumalix, dumalix.load_dumalix))
 
+    from . import malinex
+
+    def build_malinex(cfg, device=None, dtype=torch.bfloat16, seed=None):
+        if seed is not None:
+            torch.manual_seed(seed)
+        return malinex.MalinexLM(cfg, device=device, dtype=dtype)
+
+    register(malinex.ARCHITECTURE, Family(malinex.MalinexConfig, build_malinex, malinex.load_malinex))
+
 
 _register_builtin()

@@ -1,6 +1,8 @@
 """Ops of the hybrid sequence mixers: latent attention (compressed K/V cache, sliding window,
-softmax sink), the mLSTM matrix memory, the group-limited sigmoid router, and the fp32 residual
-stream of parallel layers.
+softmax sink), grouped attention over paged rows (softmax or sigmoid weights, distance penalty), the
+mLSTM matrix memory, gated linear attention, the group-limited sigmoid router and the softmax router
+with a selection bias, and the fp32 residual stream of parallel layers and of layers with a gated
+residual between two norms.
 
 GPU tensors run the HIP kernels of ``csrc/hybrid`` (``torch.ops.llmctl_hybrid.*``, library
 ``_llmctl_hybrid.so``); CPU tensors run :mod:`llmctl.ops.ref_hybrid`.  All activations are
@@ -74,7 +76,7 @@ NO_LIMIT = 1 << 30  # a window or chunk that never masks
 
 def latent_attention_prefill(qa, cache, bt, cu, ctx, window: int, sink, scale: float, rk: int, max_q: int,
                              mfma: bool = True, groups: int = 1, koff: int = 0, chunk: int = NO_LIMIT, hscale=None,
-                             ofreq=None):
+                             ofreq=None, sig_bias=None, dist_a=None, dist_b=None):
     """Prompt portions: sequence n's query rows ``[cu[n], cu[n+1])`` end at position ``ctx[n]-1``;
     ``max_q``: the longest portion (sizes the launch).  bf16 shapes that fit run on the matrix cores
     (``mfma=False`` forces the generic fp32-SIMT kernel, which also serves fp32).
@@ -84,23 +86,28 @@ def latent_attention_prefill(qa, cache, bt, cu, ctx, window: int, sink, scale: f
     are the key, its first ``rk`` entries the value.  Latent attention is ``groups=1, koff=0``.  Masks:
     ``window`` (i - j < window) and ``chunk`` (i // chunk == j // chunk), :data:`NO_LIMIT` for none.
     ``sink`` (fp32 [H] or None) joins the softmax denominator; ``hscale`` (fp32 [H]) multiplies a head's
-    scores; ``ofreq`` (fp32 [rk/2]) turns the output's neighbour pairs back by ``-position * ofreq``."""
+    scores; ``ofreq`` (fp32 [rk/2]) turns the output's neighbour pairs back by ``-position * ofreq``.
+    ``dist_a``, ``dist_b`` (fp32 [H], together): ``dist_a ln(1 + dist_b (i - j))`` is taken off the scaled score.
+    ``sig_bias`` (fp32 [H]): the weights are not a softmax; a visible key weighs ``sigmoid(score + sig_bias)``
+    and nothing is normalised over the keys (no sink then)."""
     if use_native(qa):
         return native_hybrid().latent_attn_prefill(qa, cache, bt, cu, ctx, window, sink, scale, rk, max_q, mfma, groups,
-                                                   koff, chunk, hscale, ofreq)
-    return ref.latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk, groups, koff, chunk, hscale, ofreq)
+                                                   koff, chunk, hscale, ofreq, sig_bias, dist_a, dist_b)
+    return ref.latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk, groups, koff, chunk, hscale, ofreq,
+                                sig_bias, dist_a, dist_b)
 
 
 def latent_attention_decode(qa, cache, bt, ctx, window: int, sink, scale: float, rk: int, mfma: bool = True,
                             groups: int = 1, koff: int = 0, chunk: int = NO_LIMIT, hscale=None, ofreq=None,
-                            max_ctx: int = 0):
+                            max_ctx: int = 0, sig_bias=None, dist_a=None, dist_b=None):
     """One query row per sequence, at position ``ctx[n] - 1`` (options as in the prefill form;
     ``max_ctx``: the longest context if the host knows it, it sizes the split of the keys)."""
     if use_native(qa):
         return native_hybrid().latent_attn_decode(qa, cache, bt, ctx, window, sink, scale, rk, mfma, groups, koff, chunk,
-                                                  hscale, ofreq, max_ctx)
+                                                  hscale, ofreq, max_ctx, sig_bias, dist_a, dist_b)
     cu = torch.arange(qa.shape[0] + 1, dtype=torch.int32)
-    return ref.latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk, groups, koff, chunk, hscale, ofreq)
+    return ref.latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk, groups, koff, chunk, hscale, ofreq,
+                                sig_bias, dist_a, dist_b)
 
 
 def add_rmsnorm2_f32_(x, a, b, w1, w2, eps: float, one_plus: bool, out_dtype):
@@ -151,7 +158,8 @@ def attn_qkv_prep(z, H: int, G: int, dk: int, dv: int, q_norm, k_norm, eps: floa
 
 
 def sigmoid_gate_mul(o, g):
-    """``o * sigmoid(g)`` -> g's dtype."""
+    """``o * sigmoid(g)`` -> g's dtype.  ``g`` may have fewer columns than ``o [T, C]``: ``g [T, H]`` gates
+    every run of ``C / H`` neighbouring columns (one number per head)."""
     if use_native(g):
         return native_hybrid().sigmoid_gate_mul(o, g)
     return ref.sigmoid_gate_mul(o, g)
@@ -215,11 +223,12 @@ def _mlstm_scan_chunked(q, k, v, if_raw, b_i, b_f, cap, qscale, S, n, m, state_s
     return out
 
 
-def headnorm_gate(o, w, g, eps: float, out_dtype):
-    """Per-head unit-RMS of ``o [T, H, dv]`` (fp32), times ``w [H*dv]``, times ``sigmoid(g)``."""
+def headnorm_gate(o, w, g, eps: float, out_dtype, silu: bool = False):
+    """Per-head unit-RMS of ``o [T, H, dv]`` (fp32), times ``w [H*dv]``, times ``sigmoid(g)`` (``silu``:
+    times ``g sigmoid(g)``)."""
     if use_native(o):
-        return native_hybrid().headnorm_gate(o, w, g, eps, out_dtype == torch.bfloat16)
-    return ref.headnorm_gate(o, w, g, eps, out_dtype)
+        return native_hybrid().headnorm_gate(o, w, g, eps, out_dtype == torch.bfloat16, silu)
+    return ref.headnorm_gate(o, w, g, eps, out_dtype, silu)
 
 
 def group_topk_router(logits, top: int, groups: int, keep: int):
@@ -236,3 +245,108 @@ def swiglu_any(gu):
     if use_native(gu):
         return native_hybrid().swiglu_any(gu.contiguous())
     return ref.swiglu_any(gu)
+
+
+def gated_norm_add_norm_f32_(x, y, r, w_post, w_next, eps: float, out_dtype):
+    """A sublayer's result into the fp32 residual stream of a layer with norms on both sides and a
+    gated residual, in one pass: ``g = y sigmoid(r)``; ``x += g / rms(g) * w_post`` in place; returns
+    ``x / rms(x) * w_next`` -> ``out_dtype`` (the next sublayer's input), or None when ``w_next`` is None.
+    ``y`` and ``r`` are ``[T, W]`` in the activation dtype or fp32 (row-strided views allowed)."""
+    if use_native(x):
+        h = native_hybrid().gated_norm_add_norm_f32_(x, y, r, w_post, w_next, eps, out_dtype == torch.bfloat16)
+        return h if w_next is not None else None
+    return ref.gated_norm_add_norm_f32_(x, y, r, w_post, w_next, eps, out_dtype)
+
+
+def embed_rmsnorm_f32(ids, pos, table, pos_table, w, eps: float, out_dtype):
+    """``x = table[ids] + pos_table[pos]`` (learned absolute positions) as the fp32 residual stream, and
+    its RMS norm with weight ``w`` -> ``out_dtype``.  Returns (x, h)."""
+    if use_native(table):
+        return native_hybrid().embed_rmsnorm_f32(ids, pos, table, pos_table, w, eps, out_dtype == torch.bfloat16)
+    return ref.embed_rmsnorm_f32(ids, pos, table, pos_table, w, eps, out_dtype)
+
+
+GLA_CHUNK = 64  # tokens per chunk of the chunk-parallel scan; portions of >= 4 chunks take it
+
+
+def gla_chunk_plan(cu_host, device):
+    """The chunks of a step's portions for the chunk-parallel scan, or None when no portion is long enough:
+    (chunk row offsets, first chunk of every sequence, 0 .. P-1, P zeros, P ones) on ``device`` and P.  It
+    depends on the step only, so the layers of a model share one."""
+    if cu_host is None or max((b - a for a, b in zip(cu_host[:-1], cu_host[1:])), default=0) < 4 * GLA_CHUNK:
+        return None
+    pcu, base = [0], [0]
+    for a, b in zip(cu_host[:-1], cu_host[1:]):
+        t = a
+        while t < b:
+            t = min(t + GLA_CHUNK, b)
+            pcu.append(t)
+        base.append(len(pcu) - 1)
+    P = len(pcu) - 1
+    both = torch.tensor(pcu + base, dtype=torch.int32).to(device, non_blocking=True)
+    ident = torch.arange(P, dtype=torch.int32, device=device)
+    return (both[:P + 1], both[P + 1:], ident, torch.zeros(P, dtype=torch.int32, device=device),
+            torch.ones(P, dtype=torch.int32, device=device), P)
+
+
+def gla_scan(q, k, v, z, z_bias, tau: float, qscale: float, S, state_slots, cu, start, cu_host=None, plan=None):
+    """Gated linear attention over the step's tokens: per head a memory ``S [dk, dv]`` with a decay per
+    key channel, ``a_t = sigmoid(z_t + z_bias)^(1/tau)`` (computed as ``exp(log_sigmoid / tau)`` in fp32),
+    ``S_t = diag(a_t) S_(t-1) + k_t v_t^T``, ``o_t = S_t^T (q_t qscale)``.  ``q, k [T, H, dk]``, ``v [T, H, dv]``
+    (row-strided views allowed), ``z [T, H*dk]`` fp32, ``z_bias`` fp32 ``[H*dk]``.
+    Returns fp32 ``[T, H, dv]`` and updates the state pool ``S [slots, H, dk, dv]`` in place at
+    ``state_slots[seq]`` (a sequence with ``start == 0`` begins from zeros).  ``cu_host`` (the row offsets on
+    the host) or ``plan`` (:func:`gla_chunk_plan` of them) lets long portions run chunk-parallel."""
+    if use_native(q):
+        nat = native_hybrid()
+        if plan is None and cu_host is not None:
+            plan = gla_chunk_plan(cu_host, q.device)
+        if plan is not None:
+            return _gla_scan_chunked(nat, q, k, v, z, z_bias, tau, qscale, S, state_slots, start, plan)
+        return nat.gla_scan(q, k, v, z, z_bias, tau, qscale, S, state_slots, cu, start, None, True, True)
+    return ref.gla_scan(q, k, v, z, z_bias, tau, qscale, S, state_slots, cu, start)
+
+
+def _gla_scan_chunked(nat, q, k, v, z, z_bias, tau, qscale, S, state_slots, start, plan):
+    """The same recurrence with the chunks of a portion side by side.  The memory is linear in its past:
+    over a chunk with total decay D (the product of its a_t per key channel) and own contribution S_loc (the
+    chunk run from zeros), S_end = diag(D) S_begin + S_loc.  Three passes: (1) every chunk from zeros, all at
+    once, no outputs, giving (S_loc, log D); (2) the memory at every chunk's first token, chunk after chunk
+    (elementwise), and the sequence's new carried memory; (3) every chunk again from its true memory, all at
+    once, writing outputs token by token."""
+    pcu_d, base_d, ident, zeros, ones, P = plan
+    H, dk, dv = q.shape[1], q.shape[2], v.shape[2]
+    f32 = dict(dtype=torch.float32, device=q.device)
+    loc, logd = torch.empty(P, H, dk, dv, **f32), torch.empty(P, H, dk, **f32)
+    nat.gla_scan(q, k, v, z, z_bias, tau, qscale, loc, ident, pcu_d, zeros, logd, False, True)
+    init = torch.empty_like(loc)
+    nat.gla_chunk_combine(S, state_slots, start, base_d, loc, logd, init)
+    return nat.gla_scan(q, k, v, z, z_bias, tau, qscale, init, ident, pcu_d, ones, None, True, False)
+
+
+def qk_fullnorm_prep(z, H: int, G: int, dk: int, dv: int, q_norm, k_norm, eps: float, pos, temp_coef: float,
+                     temp_every: int, cache, slots):
+    """``z [T, >= H*dk + G*dk + G*dv] = [q | k | v | ...]`` (biases already added): RMS norm over the whole
+    of q and over the whole of k before the split into heads (weights fp32 ``[H*dk]``, ``[G*dk]``); the query
+    temperature ``1 + temp_coef ln(floor((p + 1) / temp_every) + 1)`` at position p (``temp_coef`` 0: none);
+    k and v are written to the token's cache row ``[G, dv + dk] = [v | k]`` at ``slots``; returns q ``[T, H, dk]``."""
+    if use_native(z):
+        return native_hybrid().qk_fullnorm_prep(z, H, G, dk, dv, q_norm, k_norm, eps, pos, temp_coef, temp_every, cache, slots)
+    return ref.qk_fullnorm_prep(z, H, G, dk, dv, q_norm, k_norm, eps, pos, temp_coef, temp_every, cache, slots)
+
+
+def bias_topk_router(logits, bias, top: int):
+    """Softmax scores of ``logits [T, E]`` (fp32); the ``top`` experts with the largest ``score + bias`` are
+    chosen (ties: the lower index); their weights are their own scores (without the bias) over their sum
+    (+ 1e-20).  Returns (expert ids int64 [T, top], weights fp32 [T, top])."""
+    if use_native(logits):
+        return native_hybrid().bias_topk_router(logits, bias, top)
+    return ref.bias_topk_router(logits, bias, top)
+
+
+def act_any(x, kind: str):
+    """Elementwise activation of ``x`` (bf16 or fp32, computed in fp32): ``relu2`` = relu(x)^2, ``gelu`` = the
+    exact (erf) GELU."""
+    if use_native(x):
+        return native_hybrid().act_any(x, {"relu2": 0, "gelu": 1}[kind])
+    return ref.act_any(x, kind)

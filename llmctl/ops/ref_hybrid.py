@@ -61,14 +61,15 @@ def latent_q_assemble(q_lat, q, pos, inv_freq, rot_dims, dn, interleaved=False, 
 
 
 def latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk, groups=1, koff=0, chunk=1 << 30, hscale=None,
-                     ofreq=None):
+                     ofreq=None, sig_bias=None, dist_a=None, dist_b=None):
     """Attention over a paged row cache.  Sequence n owns query rows [cu[n], cu[n+1]); its last query
     sits at position ctx[n] - 1.  A token's cache row holds ``groups`` sub-rows; query head h reads
     sub-row h / (H / groups), whose entries [koff, koff + R) are the key and whose first ``rk`` entries
     are the value (latent attention: one sub-row, key = the whole row).  Position i sees j <= i inside
     its window (i - j < window) and its chunk (i // chunk == j // chunk); ``sink`` [H] joins the softmax
     denominator; ``hscale`` [H] multiplies the scores; ``ofreq`` [rk / 2] turns the output's neighbour
-    pairs back by -position * ofreq."""
+    pairs back by -position * ofreq.  ``dist_a``, ``dist_b`` [H]: ``dist_a ln(1 + dist_b (i - j))`` is taken
+    off the scaled score; ``sig_bias`` [H]: no softmax, a visible key weighs sigmoid(score + sig_bias)."""
     T, H, R = qa.shape
     bs = cache.shape[1]
     G = groups
@@ -90,6 +91,12 @@ def latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk, groups=1, 
         qpos = torch.arange(p0, ctx_l[n])
         d = qpos[:, None] - kpos[None, :]
         vis = (d >= 0) & (d < window) & (qpos[:, None] // chunk == kpos[None, :] // chunk)
+        if dist_a is not None:
+            s = s - dist_a.float().view(H, 1, 1) * torch.log1p(dist_b.float().view(H, 1, 1) * d.clamp(min=0).float())
+        if sig_bias is not None:
+            wgt = torch.sigmoid(s + sig_bias.float().view(H, 1, 1)).masked_fill(~vis, 0.0)
+            out[a:b] = torch.einsum("htk,khr->thr", wgt, rows[:, :, :rk])
+            continue
         s = s.masked_fill(~vis, float("-inf"))
         top = s.max(-1, keepdim=True).values
         if sink is not None:
@@ -167,7 +174,10 @@ def attn_qkv_prep(z, H, G, dk, dv, q_norm, k_norm, eps, pos, freq, rot_dims, int
 
 
 def sigmoid_gate_mul(o, g):
-    return (o.float() * torch.sigmoid(g.float())).to(g.dtype)
+    gate = torch.sigmoid(g.float())
+    if g.shape[-1] != o.shape[-1]:  # one gate per group of neighbouring columns
+        gate = gate.repeat_interleave(o.shape[-1] // g.shape[-1], -1)
+    return (o.float() * gate).to(g.dtype)
 
 
 def mlstm_scan(q, k, v, if_raw, b_i, b_f, cap, qscale, S, n, m, state_slots, cu, start):
@@ -203,11 +213,13 @@ def mlstm_scan(q, k, v, if_raw, b_i, b_f, cap, qscale, S, n, m, state_slots, cu,
     return out
 
 
-def headnorm_gate(o, w, g, eps, out_dtype):
+def headnorm_gate(o, w, g, eps, out_dtype, silu=False):
     T, H, dv = o.shape
     of = o.float()
     y = of * torch.rsqrt(of.pow(2).mean(-1, keepdim=True) + eps)
-    return (y.reshape(T, H * dv) * w.float() * torch.sigmoid(g.float())).to(out_dtype)
+    gf = g.float()
+    gate = gf * torch.sigmoid(gf) if silu else torch.sigmoid(gf)
+    return (y.reshape(T, H * dv) * w.float() * gate).to(out_dtype)
 
 
 def group_topk_router(logits, top, groups, keep):
@@ -226,3 +238,74 @@ def swiglu_any(gu):
     f = gu.shape[-1] // 2
     g, u = gu[..., :f].float(), gu[..., f:].float()
     return (g * torch.sigmoid(g) * u).to(gu.dtype)
+
+
+def gated_norm_add_norm_f32_(x, y, r, w_post, w_next, eps, out_dtype):
+    g = y.float() * torch.sigmoid(r.float())
+    x += g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps) * w_post.float()
+    if w_next is None:
+        return None
+    return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w_next.float()).to(out_dtype)
+
+
+def embed_rmsnorm_f32(ids, pos, table, pos_table, w, eps, out_dtype):
+    x = table[ids].float() + pos_table[pos.long()].float()
+    return x, (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+
+
+def gla_scan(q, k, v, z, z_bias, tau, qscale, S, state_slots, cu, start):
+    """Token-by-token decayed matrix memory.  The state pool S [slots, H, dk, dv] (fp32) is read at
+    ``state_slots[seq]`` (zeros when the sequence starts at position 0) and written back after the
+    sequence's last token of this step."""
+    T, H, dk = q.shape
+    dv = v.shape[-1]
+    out = torch.zeros(T, H, dv, dtype=torch.float32)
+    alpha = torch.exp(torch.nn.functional.logsigmoid(z.float() + z_bias.float()) / tau).view(T, H, dk)
+    cu_l = [int(x) for x in cu]
+    for s in range(len(cu_l) - 1):
+        a, b = cu_l[s], cu_l[s + 1]
+        if a == b:
+            continue
+        slot = int(state_slots[s])
+        Ss = torch.zeros_like(S[slot]) if int(start[s]) == 0 else S[slot].clone()
+        for t in range(a, b):
+            Ss = alpha[t][:, :, None] * Ss + k[t].float()[:, :, None] * v[t].float()[:, None, :]
+            out[t] = torch.einsum("hkv,hk->hv", Ss, q[t].float() * qscale)
+        S[slot] = Ss
+    return out
+
+
+def qk_fullnorm_prep(z, H, G, dk, dv, q_norm, k_norm, eps, pos, temp_coef, temp_every, cache, slots):
+    """z [T, >= H*dk + G*dk + G*dv] = [q | k | v | ...]: RMS norm of all of q and of all of k (weights [H*dk],
+    [G*dk]); q times 1 + temp_coef ln(floor((p + 1) / temp_every) + 1); k and v go to the token's cache row
+    [G, dv + dk] = [v | k]; returns q [T, H, dk]."""
+    T = z.shape[0]
+    zf = z.float()
+    unit = lambda x: x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    q = unit(zf[:, :H * dk]) * q_norm.float()
+    k = unit(zf[:, H * dk:(H + G) * dk]) * k_norm.float()
+    v = zf[:, (H + G) * dk:(H + G) * dk + G * dv].view(T, G, dv)
+    if temp_coef != 0.0:
+        q = q * (1.0 + temp_coef * torch.log(torch.floor((pos.float() + 1.0) / float(temp_every)) + 1.0))[:, None]
+    row = torch.cat([v, k.view(T, G, dk)], -1).reshape(T, G * (dv + dk)).to(cache.dtype)
+    ok = slots >= 0
+    cache.view(-1, cache.shape[-1])[slots[ok]] = row[ok]
+    return q.view(T, H, dk).to(z.dtype)
+
+
+def bias_topk_router(logits, bias, top):
+    s = torch.softmax(logits.float(), -1)
+    idx = (s + bias.float()).topk(top, -1).indices
+    w = s.gather(1, idx)
+    return idx, w / (w.sum(-1, keepdim=True) + 1e-20)
+
+
+def act_any(x, kind):
+    xf = x.float()
+    if kind == "relu2":
+        y = torch.relu(xf).pow(2)
+    elif kind == "gelu":
+        y = 0.5 * xf * (1.0 + torch.erf(xf * 0.7071067811865476))
+    else:
+        raise ValueError(f"unknown activation {kind!r}")
+    return y.to(x.dtype)

@@ -216,6 +216,9 @@ class InferenceEngine:
                               np.asarray(dp["positions"], dtype=np.int32) if Td else np.zeros(0, np.int32)])
         slots = np.concatenate([np.asarray(pp["slots"], dtype=np.int64) if Tp else np.zeros(0, np.int64),
                                 np.asarray(dp["slots"], dtype=np.int64) if Td else np.zeros(0, np.int64)])
+        limit = getattr(self.model, "position_limit", None)  # models with a table of learned positions
+        if limit is not None and len(pos) and int(pos.max()) >= limit:
+            raise ValueError(f"position {int(pos.max())} is beyond the model's {limit} learned positions")
         p_cu = list(pp["cu"]) if Tp else [0]
         cu = p_cu + [Tp + i + 1 for i in range(Td)]
         start = ([c - (b - a) for a, b, c in zip(p_cu[:-1], p_cu[1:], pp["ctx"])] if Tp else []) + (
