@@ -112,6 +112,9 @@ struct RowAttnOpts {
   const float* hscale = nullptr;      // [H] a factor on every head's scores
   const float* ofreq = nullptr;       // [rk / 2] turn the output's neighbour pairs back by -position * ofreq
   int64_t max_ctx = 0;                // the longest context of the step, if the host knows it (sizes decode splits)
+  const float* dist_a = nullptr;      // [H], with dist_b [H]: dist_a ln(1 + dist_b (i - j)) is taken off the scaled score
+  const float* dist_b = nullptr;
+  const float* sig_bias = nullptr;    // [H]: no softmax; a visible key weighs sigmoid(score + sig_bias), nothing is normalised
 };
 
 }  // namespace llmctl_hybrid

@@ -93,6 +93,9 @@ struct GenArgs {
   const float* sink;    // nullptr: none
   const float* hscale;  // nullptr: 1
   const float* ofreq;   // nullptr: the output is not turned back
+  const float* dist_a;  // nullptr: no distance penalty
+  const float* dist_b;
+  const float* sig_bias;  // SIG forms: the head's bias inside the sigmoid
   int bt_stride, H, R, rk, bs, window, chunk, G, rs, koff;
   float scale;
 };
@@ -100,7 +103,8 @@ struct GenArgs {
 __device__ __forceinline__ int first_visible(int p, int window, int chunk) { return max(max(p - window + 1, (p / chunk) * chunk), 0); }
 
 // grid (q tiles of 64, sequences, heads * value tiles); one wave per block, lane = query.
-template <typename T, int VT>
+// SIG: a visible key weighs sigmoid(score + bias) and nothing is normalised (no running maximum, no sink).
+template <typename T, int VT, bool SIG>
 __global__ __launch_bounds__(64) void latent_attn_prefill_kernel(const T* __restrict__ qa, const T* __restrict__ cache, const int* __restrict__ cu,
                                                                  T* __restrict__ out, GenArgs g, int nvt) {
   extern __shared__ float qT[];  // [R][64]
@@ -120,6 +124,9 @@ __global__ __launch_bounds__(64) void latent_attn_prefill_kernel(const T* __rest
   const int j0 = first_visible(p0 + q0, g.window, g.chunk);
   const int lo = first_visible(qp, g.window, g.chunk);
   const float scale = g.scale * (g.hscale != nullptr ? g.hscale[h] : 1.0f);
+  const bool pen = g.dist_a != nullptr;
+  const float da = pen ? g.dist_a[h] : 0.f, db = pen ? g.dist_b[h] : 0.f;
+  const float sb = SIG ? g.sig_bias[h] : 0.f;
   float m = -INFINITY, l = 0.f;
   if (g.sink != nullptr) {  // the sink: exp(sink - m) with m = sink
     m = g.sink[h];
@@ -137,16 +144,23 @@ __global__ __launch_bounds__(64) void latent_attn_prefill_kernel(const T* __rest
     for (int d = 0; d < R; ++d) s += qT[d * 64 + lane] * ldf(key + d);
     s *= scale;
     if (live && j <= qp && j >= lo) {
-      const float mn = fmaxf(m, s);
-      const float corr = expf(m - mn), p = expf(s - mn);  // m = -inf before the first key: corr = 0
-      l = l * corr + p;
+      if (pen) s -= da * log1pf(db * (float)(qp - j));
+      if constexpr (SIG) {
+        const float p = 1.0f / (1.0f + expf(-(s + sb)));
 #pragma unroll
-      for (int i = 0; i < VT; ++i) acc[i] = acc[i] * corr + p * ldf(row + min(v0 + i, rk - 1));
-      m = mn;
+        for (int i = 0; i < VT; ++i) acc[i] += p * ldf(row + min(v0 + i, rk - 1));
+      } else {
+        const float mn = fmaxf(m, s);
+        const float corr = expf(m - mn), p = expf(s - mn);  // m = -inf before the first key: corr = 0
+        l = l * corr + p;
+#pragma unroll
+        for (int i = 0; i < VT; ++i) acc[i] = acc[i] * corr + p * ldf(row + min(v0 + i, rk - 1));
+        m = mn;
+      }
     }
   }
   if (!live) return;
-  const float inv = 1.0f / l;
+  const float inv = SIG ? 1.0f : 1.0f / l;
   if (g.ofreq != nullptr) {  // neighbour pairs (2m, 2m + 1) turned back by the query's position
 #pragma unroll
     for (int i = 0; i < VT; i += 2)
@@ -166,7 +180,7 @@ __global__ __launch_bounds__(64) void latent_attn_prefill_kernel(const T* __rest
 
 // ----------------------------------------------------------------------------------------- decode
 // grid (sequences, heads); 4 waves, each takes chunks of 64 keys (one key per lane for the score).
-template <typename T, int NA>
+template <typename T, int NA, bool SIG>
 __global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __restrict__ qa, const T* __restrict__ cache, T* __restrict__ out,
                                                                  GenArgs g) {
   extern __shared__ float sm[];
@@ -187,7 +201,10 @@ __global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __rest
   const int* btn = g.bt + (int64_t)n * g.bt_stride;
   const int grp = h / (H / g.G);
   const float scale = g.scale * (g.hscale != nullptr ? g.hscale[h] : 1.0f);
-  float m = -INFINITY, l = 0.f;
+  const bool pen = g.dist_a != nullptr;
+  const float da = pen ? g.dist_a[h] : 0.f, db = pen ? g.dist_b[h] : 0.f;
+  const float sb = SIG ? g.sig_bias[h] : 0.f;
+  float m = SIG ? 0.f : -INFINITY, l = 0.f;
   float acc[NA];
 #pragma unroll
   for (int i = 0; i < NA; ++i) acc[i] = 0.f;
@@ -202,12 +219,20 @@ __global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __rest
       float d0 = 0.f;
       for (int d = 0; d < R; ++d) d0 += qs[d] * ldf(key + d);
       s = d0 * scale;
+      if (pen) s -= da * log1pf(db * (float)(len - 1 - j));
     }
-    const float mn = fmaxf(m, wave_max(s));  // at least one key of the chunk is valid: finite
-    const float p = ok ? expf(s - mn) : 0.f;
-    const float corr = expf(m - mn);         // m = -inf on the first chunk: 0
-    l = l * corr + wave_sum(p);
-    m = mn;
+    float p, corr;
+    if constexpr (SIG) {
+      p = ok ? 1.0f / (1.0f + expf(-(s + sb))) : 0.f;
+      corr = 1.0f;
+      l = 1.0f;  // the waves' parts are summed as they are
+    } else {
+      const float mn = fmaxf(m, wave_max(s));  // at least one key of the chunk is valid: finite
+      p = ok ? expf(s - mn) : 0.f;
+      corr = expf(m - mn);                     // m = -inf on the first chunk: 0
+      l = l * corr + wave_sum(p);
+      m = mn;
+    }
     pw[wave * 64 + lane] = p;
     ro[wave * 64 + lane] = slot;
     __builtin_amdgcn_wave_barrier();
@@ -244,6 +269,11 @@ __global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __rest
   for (int w = 0; w < 4; ++w) {
     f[w] = ml[w * 2 + 1] > 0.f ? expf(ml[w * 2] - M) : 0.f;
     L += ml[w * 2 + 1] * f[w];
+  }
+  if constexpr (SIG) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) f[w] = 1.0f;  // (a wave that saw no key holds zeros)
+    L = 1.0f;
   }
   T* o = out + ((int64_t)n * H + h) * rk;
   for (int d = threadIdx.x; d < rk; d += 256) {
@@ -325,7 +355,8 @@ at::Tensor latent_q_assemble(const at::Tensor& q_lat, const at::Tensor& q, const
 // The optional tensors of the general form, checked; returns the kernels' view of them.
 static RowAttnOpts row_opts(const at::Tensor& qa, const at::Tensor& cache, int64_t rk, const c10::optional<at::Tensor>& sink, int64_t groups,
                             int64_t koff, int64_t chunk, const c10::optional<at::Tensor>& hscale, const c10::optional<at::Tensor>& ofreq,
-                            int64_t max_ctx, const float** sink_p) {
+                            int64_t max_ctx, const float** sink_p, const c10::optional<at::Tensor>& sig_bias = c10::nullopt,
+                            const c10::optional<at::Tensor>& dist_a = c10::nullopt, const c10::optional<at::Tensor>& dist_b = c10::nullopt) {
   const int64_t H = qa.size(1), R = qa.size(2);
   HYB_CHECK(groups >= 1 && H % groups == 0 && cache.size(2) % groups == 0, "kv groups must divide the heads and the cache row");
   const int64_t rs = cache.size(2) / groups;
@@ -342,6 +373,12 @@ static RowAttnOpts row_opts(const at::Tensor& qa, const at::Tensor& cache, int64
   x.hscale = hscale.has_value() ? hscale->data_ptr<float>() : nullptr;
   x.ofreq = ofreq.has_value() ? ofreq->data_ptr<float>() : nullptr;
   x.max_ctx = max_ctx;
+  HYB_CHECK(dist_a.has_value() == dist_b.has_value(), "the distance penalty takes both of its vectors");
+  if (dist_a.has_value()) HYB_CHECK(f32_vec(*dist_a, H) && f32_vec(*dist_b, H), "distance penalty: fp32 [H] twice");
+  if (sig_bias.has_value()) HYB_CHECK(f32_vec(*sig_bias, H) && !sink.has_value() && !ofreq.has_value(), "sigmoid weights: fp32 bias [H], no sink, no output turn");
+  x.dist_a = dist_a.has_value() ? dist_a->data_ptr<float>() : nullptr;
+  x.dist_b = dist_b.has_value() ? dist_b->data_ptr<float>() : nullptr;
+  x.sig_bias = sig_bias.has_value() ? sig_bias->data_ptr<float>() : nullptr;
   return x;
 }
 
@@ -353,6 +390,9 @@ static GenArgs gen_args(const at::Tensor& qa, const at::Tensor& cache, const at:
   g.sink = sink;
   g.hscale = x.hscale;
   g.ofreq = x.ofreq;
+  g.dist_a = x.dist_a;
+  g.dist_b = x.dist_b;
+  g.sig_bias = x.sig_bias;
   g.bt_stride = (int)bt.size(1);
   g.H = (int)qa.size(1);
   g.R = (int)qa.size(2);
@@ -370,7 +410,9 @@ static GenArgs gen_args(const at::Tensor& qa, const at::Tensor& cache, const at:
 at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor& cu,
                                const at::Tensor& ctx, int64_t window, const c10::optional<at::Tensor>& sink, double scale, int64_t rk,
                                int64_t max_q, bool mfma, int64_t groups, int64_t koff, int64_t chunk,
-                               const c10::optional<at::Tensor>& hscale, const c10::optional<at::Tensor>& ofreq) {
+                               const c10::optional<at::Tensor>& hscale, const c10::optional<at::Tensor>& ofreq,
+                               const c10::optional<at::Tensor>& sig_bias, const c10::optional<at::Tensor>& dist_a,
+                               const c10::optional<at::Tensor>& dist_b) {
   HYB_CHECK(qa.is_cuda() && qa.is_contiguous() && qa.dim() == 3, "qa: contiguous [T, H, R]");
   const int64_t T = qa.size(0), H = qa.size(1), R = qa.size(2);
   check_cache(cache, qa, cache.size(2));
@@ -382,12 +424,12 @@ at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, co
   HYB_CHECK(window >= 1 && max_q >= 1, "window >= 1, max_q >= 1");
   window = std::min<int64_t>(window, (int64_t)1 << 30);
   const float* sink_p;
-  const RowAttnOpts x = row_opts(qa, cache, rk, sink, groups, koff, chunk, hscale, ofreq, 0, &sink_p);
+  const RowAttnOpts x = row_opts(qa, cache, rk, sink, groups, koff, chunk, hscale, ofreq, 0, &sink_p, sig_bias, dist_a, dist_b);
   HYB_CHECK((size_t)R * 64 * sizeof(float) <= 160 * 1024, "key too wide for the query tile in LDS");
   c10::DeviceGuard guard(qa.device());
   at::Tensor out = at::empty({T, H, rk}, qa.options());
   if (T == 0 || ns == 0) return out;
-  if (mfma && latent_attn_mfma_ok(qa, rk, cache.size(2) / groups, koff, x.ofreq != nullptr)) {
+  if (mfma && (x.dist_a == nullptr || x.sig_bias != nullptr) && latent_attn_mfma_ok(qa, rk, cache.size(2) / groups, koff, x.ofreq != nullptr || x.sig_bias != nullptr)) {
     latent_attn_mfma(qa, cache, bt, &cu, ctx, window, sink_p, scale, rk, max_q, out, x);
     return out;
   }
@@ -403,9 +445,15 @@ at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, co
       if (lds > 64 * 1024) HYB_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess, "LDS size");
       kern<<<grid, 64, lds, cur_stream()>>>((const Tt*)qa.data_ptr(), (const Tt*)cache.data_ptr(), cu.data_ptr<int>(), (Tt*)out.data_ptr(), g, nvt);
     };
-    if (VT == 32) launch(latent_attn_prefill_kernel<Tt, 32>);
-    else if (VT == 64) launch(latent_attn_prefill_kernel<Tt, 64>);
-    else launch(latent_attn_prefill_kernel<Tt, 128>);
+    if (x.sig_bias != nullptr) {
+      if (VT == 32) launch(latent_attn_prefill_kernel<Tt, 32, true>);
+      else if (VT == 64) launch(latent_attn_prefill_kernel<Tt, 64, true>);
+      else launch(latent_attn_prefill_kernel<Tt, 128, true>);
+    } else {
+      if (VT == 32) launch(latent_attn_prefill_kernel<Tt, 32, false>);
+      else if (VT == 64) launch(latent_attn_prefill_kernel<Tt, 64, false>);
+      else launch(latent_attn_prefill_kernel<Tt, 128, false>);
+    }
   });
   return out;
 }
@@ -413,7 +461,8 @@ at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, co
 at::Tensor latent_attn_decode(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor& ctx,
                               int64_t window, const c10::optional<at::Tensor>& sink, double scale, int64_t rk, bool mfma, int64_t groups,
                               int64_t koff, int64_t chunk, const c10::optional<at::Tensor>& hscale, const c10::optional<at::Tensor>& ofreq,
-                              int64_t max_ctx) {
+                              int64_t max_ctx, const c10::optional<at::Tensor>& sig_bias, const c10::optional<at::Tensor>& dist_a,
+                              const c10::optional<at::Tensor>& dist_b) {
   HYB_CHECK(qa.is_cuda() && qa.is_contiguous() && qa.dim() == 3, "qa: contiguous [n, H, R]");
   const int64_t ns = qa.size(0), H = qa.size(1), R = qa.size(2);
   check_cache(cache, qa, cache.size(2));
@@ -423,11 +472,11 @@ at::Tensor latent_attn_decode(const at::Tensor& qa, const at::Tensor& cache, con
   HYB_CHECK(window >= 1, "window >= 1");
   window = std::min<int64_t>(window, (int64_t)1 << 30);
   const float* sink_p;
-  const RowAttnOpts x = row_opts(qa, cache, rk, sink, groups, koff, chunk, hscale, ofreq, max_ctx, &sink_p);
+  const RowAttnOpts x = row_opts(qa, cache, rk, sink, groups, koff, chunk, hscale, ofreq, max_ctx, &sink_p, sig_bias, dist_a, dist_b);
   c10::DeviceGuard guard(qa.device());
   at::Tensor out = at::empty({ns, H, rk}, qa.options());
   if (ns == 0) return out;
-  if (mfma && latent_attn_mfma_ok(qa, rk, cache.size(2) / groups, koff, x.ofreq != nullptr)) {
+  if (mfma && (x.dist_a == nullptr || x.sig_bias != nullptr) && latent_attn_mfma_ok(qa, rk, cache.size(2) / groups, koff, x.ofreq != nullptr || x.sig_bias != nullptr)) {
     latent_attn_mfma(qa, cache, bt, nullptr, ctx, window, sink_p, scale, rk, 1, out, x);
     return out;
   }
@@ -439,10 +488,14 @@ at::Tensor latent_attn_decode(const at::Tensor& qa, const at::Tensor& cache, con
   const GenArgs g = gen_args(qa, cache, bt, ctx, sink_p, window, scale, rk, x);
   dispatch_act(qa, [&](auto* tag) {
     using Tt = std::remove_pointer_t<decltype(tag)>;
-    if (rk <= 128)
-      latent_attn_decode_kernel<Tt, 2><<<grid, 256, lds, cur_stream()>>>((const Tt*)qa.data_ptr(), (const Tt*)cache.data_ptr(), (Tt*)out.data_ptr(), g);
-    else
-      latent_attn_decode_kernel<Tt, 8><<<grid, 256, lds, cur_stream()>>>((const Tt*)qa.data_ptr(), (const Tt*)cache.data_ptr(), (Tt*)out.data_ptr(), g);
+    auto launch = [&](auto kern) { kern<<<grid, 256, lds, cur_stream()>>>((const Tt*)qa.data_ptr(), (const Tt*)cache.data_ptr(), (Tt*)out.data_ptr(), g); };
+    if (x.sig_bias != nullptr) {
+      if (rk <= 128) launch(latent_attn_decode_kernel<Tt, 2, true>);
+      else launch(latent_attn_decode_kernel<Tt, 8, true>);
+    } else {
+      if (rk <= 128) launch(latent_attn_decode_kernel<Tt, 2, false>);
+      else launch(latent_attn_decode_kernel<Tt, 8, false>);
+    }
   });
   return out;
 }

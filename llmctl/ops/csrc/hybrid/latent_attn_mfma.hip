@@ -37,6 +37,9 @@ struct LArgs {
   const float* sink;    // nullptr: no sink
   const float* hscale;  // nullptr or a factor on every head's scores
   const float* ofreq;   // nullptr, or [rk / 2]: the output's neighbour pairs are turned back by -position * ofreq
+  const float* dist_a;  // SIG forms: [H] each; dist_a ln(1 + dist_b (i - j)) is taken off the scaled score and a visible
+  const float* dist_b;  // key weighs sigmoid(score + sig_bias); dist_a may be nullptr (no penalty)
+  const float* sig_bias;
   int H, R, rk, bs, maxb, window, HB, nvt;
   int G, rs, koff, chunk, hpg;  // kv groups, row width, key's first column, chunk mask size, head tiles per group
   float scale_log2;
@@ -48,8 +51,10 @@ struct LArgs {
 };
 
 // ROT: the output's neighbour pairs are turned back by the query's position (a.ofreq); a template flag
-// so that the forms without it keep their register budget
-template <int NCB, int NDB, bool ROT>
+// so that the forms without it keep their register budget.  SIG: the weights are sigmoids of the scores
+// (after the distance penalty), not a softmax: no running maximum, no rescale, no denominator; the splits
+// of decode rows are merged as a plain sum (m = 0 everywhere, l = 1 in the first split only).
+template <int NCB, int NDB, bool ROT, bool SIG = false>
 __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   constexpr int NKS = NCB * 8;
   constexpr int NTB = (NDB + 3) / 4;
@@ -107,6 +112,13 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   if (split > 0) {                                 // (the sink is counted by the first split only)
     m_i = -INFINITY;
     l_i = 0.f;
+  }
+  float pen_a = 0.f, pen_b = 0.f, sig_b2 = 0.f;
+  if constexpr (SIG) {
+    m_i = 0.f;
+    l_i = split == 0 ? 1.f : 0.f;
+    if (a.dist_a != nullptr) pen_a = a.dist_a[headc], pen_b = a.dist_b[headc];
+    sig_b2 = a.sig_bias[headc] * kLog2e;
   }
 
   const int first_pos = pos0 + tok0, last_pos = pos0 + min(tok0 + TB, qlen) - 1;
@@ -210,58 +222,76 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
         s[kb] = mfma32(kf, qf[ks], s[kb]);
       }
     }
-    float mx = -INFINITY;
-    if (kv0 + LKB - 1 <= w_first && kv0 >= w_lo_last && kv0 + LKB - 1 < ctx) {
-      // every key of the tile is visible to every row of this wave: no mask (rows past the portion's end
-      // carry finite scores of a repeated row and are never stored)
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          s[kb][i] *= my_scale;
-          mx = fmaxf(mx, s[kb][i]);
-        }
-      if (!valid) mx = -INFINITY;  // such a row must not trigger the wave's rescale
-    } else {
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          float x = s[kb][i] * my_scale;
-          const int key = kv0 + kb * 32 + acc_row(i, hh);
-          if (!valid || key > my_pos || key < my_lo || key >= ctx) x = -INFINITY;
-          s[kb][i] = x;
-          mx = fmaxf(mx, x);
-        }
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const bool grow = __builtin_amdgcn_ballot_w64(mx > m_i + kRescaleTh) != 0;
-    const float m_raw = grow ? fmaxf(m_i, mx) : m_i;
-    const float m_new = m_raw == -INFINITY ? 0.f : m_raw;  // nothing seen yet (a later split, all keys masked)
-    float rs = 0.f;
     bf16x8_t pb[2][2];
+    if constexpr (SIG) {
+      // x (log2 domain) = s * scale - a log2(1 + b (i - j)) + bias; weight = 1 / (1 + 2^-x); hidden keys weigh 0
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      float p[16];
+      for (int kb = 0; kb < 2; ++kb) {
+        float p[16];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        p[i] = fast_exp2(s[kb][i] - m_new);
-        rs += p[i];
+        for (int i = 0; i < 16; ++i) {
+          const int key = kv0 + kb * 32 + acc_row(i, hh);
+          const float dist = (float)max(my_pos - key, 0);
+          const float x = s[kb][i] * my_scale - pen_a * __log2f(1.0f + pen_b * dist) + sig_b2;
+          const float w = __builtin_amdgcn_rcpf(1.0f + fast_exp2(-x));
+          p[i] = (!valid || key > my_pos || key < my_lo || key >= ctx) ? 0.f : w;
+        }
+        pb[kb][0] = to_bf16x8(p);
+        pb[kb][1] = to_bf16x8(p + 8);
       }
-      pb[kb][0] = to_bf16x8(p);
-      pb[kb][1] = to_bf16x8(p + 8);
-    }
-    rs += __shfl_xor(rs, 32);
-    if (grow) {
-      const float alpha = fast_exp2(m_i - m_new);
-      l_i *= alpha;
+    } else {
+      float mx = -INFINITY;
+      if (kv0 + LKB - 1 <= w_first && kv0 >= w_lo_last && kv0 + LKB - 1 < ctx) {
+        // every key of the tile is visible to every row of this wave: no mask (rows past the portion's end
+        // carry finite scores of a repeated row and are never stored)
 #pragma unroll
-      for (int d = 0; d < NDB; ++d)
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) o[d][i] *= alpha;
+          for (int i = 0; i < 16; ++i) {
+            s[kb][i] *= my_scale;
+            mx = fmaxf(mx, s[kb][i]);
+          }
+        if (!valid) mx = -INFINITY;  // such a row must not trigger the wave's rescale
+      } else {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            float x = s[kb][i] * my_scale;
+            const int key = kv0 + kb * 32 + acc_row(i, hh);
+            if (!valid || key > my_pos || key < my_lo || key >= ctx) x = -INFINITY;
+            s[kb][i] = x;
+            mx = fmaxf(mx, x);
+          }
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const bool grow = __builtin_amdgcn_ballot_w64(mx > m_i + kRescaleTh) != 0;
+      const float m_raw = grow ? fmaxf(m_i, mx) : m_i;
+      const float m_new = m_raw == -INFINITY ? 0.f : m_raw;  // nothing seen yet (a later split, all keys masked)
+      float rs = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        float p[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          p[i] = fast_exp2(s[kb][i] - m_new);
+          rs += p[i];
+        }
+        pb[kb][0] = to_bf16x8(p);
+        pb[kb][1] = to_bf16x8(p + 8);
+      }
+      rs += __shfl_xor(rs, 32);
+      if (grow) {
+        const float alpha = fast_exp2(m_i - m_new);
+        l_i *= alpha;
+#pragma unroll
+        for (int d = 0; d < NDB; ++d)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[d][i] *= alpha;
+      }
+      l_i += rs;
+      m_i = m_raw;
     }
-    l_i += rs;
-    m_i = m_raw;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -344,7 +374,7 @@ __global__ void latent_split_merge_kernel(const float* __restrict__ ws_o, const 
   }
 }
 
-template <int NCB, bool ROT>
+template <int NCB, bool ROT, bool SIG = false>
 void launch_ncb(const LArgs& a, int ndb, dim3 grid, hipStream_t st) {
   auto go = [&](auto kern, int NDBv) {
     const size_t one = (size_t)(NCB + (NDBv + 3) / 4) * LIMG;
@@ -352,13 +382,14 @@ void launch_ncb(const LArgs& a, int ndb, dim3 grid, hipStream_t st) {
     HYB_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess, "LDS size");
     kern<<<grid, 256, lds, st>>>(a);
   };
-  if (ndb == 2) go(latent_attn_mfma_kernel<NCB, 2, ROT>, 2);
-  else if (ndb == 4) go(latent_attn_mfma_kernel<NCB, 4, ROT>, 4);
-  else go(latent_attn_mfma_kernel<NCB, 8, ROT>, 8);
+  if (ndb == 2) go(latent_attn_mfma_kernel<NCB, 2, ROT, SIG>, 2);
+  else if (ndb == 4) go(latent_attn_mfma_kernel<NCB, 4, ROT, SIG>, 4);
+  else go(latent_attn_mfma_kernel<NCB, 8, ROT, SIG>, 8);
 }
 }  // namespace
 
-// turn_back: the output is to be turned back (RowAttnOpts::ofreq); built for keys up to 256 wide
+// turn_back: the output is to be turned back (RowAttnOpts::ofreq) or the weights are sigmoids
+// (RowAttnOpts::sig_bias); those forms are built for keys up to 256 wide
 bool latent_attn_mfma_ok(const at::Tensor& qa, int64_t rk, int64_t rs, int64_t koff, bool turn_back) {
   const int64_t R = qa.size(2);
   return qa.scalar_type() == at::kBFloat16 && R % 8 == 0 && rk % 8 == 0 && rs % 8 == 0 && koff % 8 == 0 && R <= (turn_back ? 256 : 640) && qa.size(1) >= 1;
@@ -395,13 +426,16 @@ void latent_attn_mfma(const at::Tensor& qa, const at::Tensor& cache, const at::T
   }
   LArgs a{reinterpret_cast<const unsigned short*>(qa.data_ptr()), reinterpret_cast<const unsigned short*>(cache.data_ptr()),
           reinterpret_cast<unsigned short*>(out.data_ptr()), bt.data_ptr<int>(), cu ? cu->data_ptr<int>() : nullptr, ctx.data_ptr<int>(),
-          sink, x.hscale, x.ofreq, (int)H, (int)R, (int)rk, (int)cache.size(1), (int)bt.size(1), (int)window, HB, nvt,
+          sink, x.hscale, x.ofreq, x.dist_a, x.dist_b, x.sig_bias, (int)H, (int)R, (int)rk, (int)cache.size(1), (int)bt.size(1), (int)window, HB, nvt,
           (int)G, (int)rs, (int)x.koff, (int)x.chunk, hpg,
           (float)(scale * 1.4426950408889634), nsplit, nsplit > 1 ? ws_o.data_ptr<float>() : nullptr,
           nsplit > 1 ? ws_ml.data_ptr<float>() : nullptr};
   dim3 grid(nsplit > 1 ? (unsigned)nsplit : (unsigned)((max_q + TB - 1) / TB), (unsigned)ns, (unsigned)(hgroups * nvt));
   hipStream_t st = cur_stream();
-  if (x.ofreq != nullptr) {
+  if (x.sig_bias != nullptr) {  // built for keys up to 256 wide (latent_attn_mfma_ok)
+    if (ncb == 1) launch_ncb<1, false, true>(a, ndb, grid, st);
+    else launch_ncb<2, false, true>(a, ndb, grid, st);
+  } else if (x.ofreq != nullptr) {
     if (ncb == 1) launch_ncb<1, true>(a, ndb, grid, st);
     else launch_ncb<2, true>(a, ndb, grid, st);
   } else {

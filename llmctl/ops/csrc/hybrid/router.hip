@@ -77,4 +77,57 @@ std::tuple<at::Tensor, at::Tensor> group_topk_router(const at::Tensor& logits, i
   return {idx, wgt};
 }
 
+// Softmax router with a selection bias: s = softmax(logits) (fp32); the ``top`` experts with the largest
+// s + bias are chosen (ties: the lower index); their weights are their own s over the sum of the chosen
+// ones (+ 1e-20).  One thread per token.
+__global__ void bias_topk_router_kernel(const float* __restrict__ logits, const float* __restrict__ bias, int64_t* __restrict__ idx,
+                                        float* __restrict__ wgt, int64_t T, int E, int top) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const float* z = logits + t * E;
+  float mx = -INFINITY;
+  for (int e = 0; e < E; ++e) mx = fmaxf(mx, z[e]);
+  float den = 0.f;
+  for (int e = 0; e < E; ++e) den += expf(z[e] - mx);
+  const float inv = 1.0f / den;
+  int esel[MAXPICK];
+  float sum = 0.f;
+  for (int kk = 0; kk < top; ++kk) {
+    float best = -INFINITY, bs = 0.f;
+    int bi = -1;
+    for (int e = 0; e < E; ++e) {
+      bool used = false;
+      for (int w = 0; w < kk; ++w) used |= esel[w] == e;
+      if (used) continue;
+      const float s = expf(z[e] - mx) * inv;
+      const float c = s + bias[e];
+      if (bi < 0 || c > best) {
+        best = c;
+        bs = s;
+        bi = e;
+      }
+    }
+    esel[kk] = bi;
+    idx[t * top + kk] = bi;
+    wgt[t * top + kk] = bs;
+    sum += bs;
+  }
+  const float norm = 1.0f / (sum + 1e-20f);
+  for (int kk = 0; kk < top; ++kk) wgt[t * top + kk] *= norm;
+}
+
+std::tuple<at::Tensor, at::Tensor> bias_topk_router(const at::Tensor& logits, const at::Tensor& bias, int64_t top) {
+  HYB_CHECK(logits.is_cuda() && logits.is_contiguous() && logits.dim() == 2 && logits.scalar_type() == at::kFloat, "logits: contiguous fp32 [T, E]");
+  const int64_t T = logits.size(0), E = logits.size(1);
+  HYB_CHECK(bias.is_cuda() && bias.is_contiguous() && bias.scalar_type() == at::kFloat && bias.numel() == E, "bias: fp32 [E]");
+  HYB_CHECK(top >= 1 && top <= E && top <= MAXPICK, "top in 1 .. min(E, 64)");
+  c10::DeviceGuard guard(logits.device());
+  at::Tensor idx = at::empty({T, top}, logits.options().dtype(at::kLong));
+  at::Tensor wgt = at::empty({T, top}, logits.options());
+  if (T == 0) return {idx, wgt};
+  bias_topk_router_kernel<<<dim3((unsigned)((T + 127) / 128)), 128, 0, cur_stream()>>>(logits.data_ptr<float>(), bias.data_ptr<float>(),
+                                                                                      idx.data_ptr<int64_t>(), wgt.data_ptr<float>(), T, (int)E, (int)top);
+  return {idx, wgt};
+}
+
 }  // namespace llmctl_hybrid

@@ -145,12 +145,12 @@ __global__ __launch_bounds__(NT) void rmsnorm_cols_kernel(const T* __restrict__ 
 
 template <typename TO, typename TG>
 __global__ void gate_mul_kernel(const TO* __restrict__ o, const TG* __restrict__ g, int64_t g_stride, TG* __restrict__ y,
-                                int64_t rows, int N) {
+                                int64_t rows, int N, int per) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= rows * N) return;
   const int64_t r = i / N;
   const int c = (int)(i - r * N);
-  const float gv = ldf(g + r * g_stride + c);
+  const float gv = ldf(g + r * g_stride + c / per);  // one gate per ``per`` neighbouring columns
   stf(y + i, ldf(o + i) * (1.0f / (1.0f + expf(-gv))));
 }
 
@@ -164,11 +164,11 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ y, int64
   stf(y + i, g / (1.0f + expf(-g)) * u);
 }
 
-// o [T, H, dv] fp32 -> y [T, H*dv]: o / rms(o over dv) * w * sigmoid(g); one wave per (token, head).
+// o [T, H, dv] fp32 -> y [T, H*dv]: o / rms(o over dv) * w * sigmoid(g) (silu: * g sigmoid(g)); one wave per (token, head).
 template <typename T>
 __global__ __launch_bounds__(NT) void headnorm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w,
                                                            const T* __restrict__ g, int64_t g_stride, T* __restrict__ y,
-                                                           int64_t pairs, int H, int dv, float eps) {
+                                                           int64_t pairs, int H, int dv, float eps, int silu) {
   const int64_t p = (int64_t)blockIdx.x * NW + (threadIdx.x >> 6);
   if (p >= pairs) return;
   const int lane = threadIdx.x & 63;
@@ -180,7 +180,8 @@ __global__ __launch_bounds__(NT) void headnorm_gate_kernel(const float* __restri
   const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)dv + eps);
   for (int c = lane; c < dv; c += 64) {
     const float gv = ldf(g + t * g_stride + hd * dv + c);
-    stf(y + p * dv + c, op[c] * rstd * w[hd * dv + c] * (1.0f / (1.0f + expf(-gv))));
+    const float gate = 1.0f / (1.0f + expf(-gv));
+    stf(y + p * dv + c, op[c] * rstd * w[hd * dv + c] * (silu ? gv * gate : gate));
   }
 }
 
@@ -258,16 +259,17 @@ at::Tensor rmsnorm_cols(const at::Tensor& x, const at::Tensor& w, double eps, in
 
 at::Tensor sigmoid_gate_mul(const at::Tensor& o, const at::Tensor& g) {
   check_rows(g, "g");
-  HYB_CHECK(o.is_cuda() && o.is_contiguous() && o.dim() == 2 && o.sizes() == g.sizes(), "o: contiguous, g's shape");
+  HYB_CHECK(o.is_cuda() && o.is_contiguous() && o.dim() == 2 && o.size(0) == g.size(0) && g.size(1) >= 1 && o.size(1) % g.size(1) == 0,
+            "o: contiguous [T, C]; g [T, C] or [T, H] with H dividing C");
   HYB_CHECK(o.scalar_type() == g.scalar_type(), "o and g share a dtype");
   c10::DeviceGuard guard(g.device());
-  at::Tensor y = at::empty(g.sizes(), g.options());
-  const int64_t n = g.numel();
+  at::Tensor y = at::empty(o.sizes(), g.options());
+  const int64_t n = o.numel();
   if (n == 0) return y;
   dispatch_act(g, [&](auto* tag) {
     using T = std::remove_pointer_t<decltype(tag)>;
     gate_mul_kernel<T, T><<<dim3((unsigned)((n + 255) / 256)), 256, 0, cur_stream()>>>((const T*)o.data_ptr(), (const T*)g.data_ptr(),
-                                                                                     g.stride(0), (T*)y.data_ptr(), g.size(0), (int)g.size(1));
+                                                                                     g.stride(0), (T*)y.data_ptr(), o.size(0), (int)o.size(1), (int)(o.size(1) / g.size(1)));
   });
   return y;
 }
@@ -358,7 +360,7 @@ at::Tensor clamped_glu(const at::Tensor& gu, double limit, double alpha) {
   return y;
 }
 
-at::Tensor headnorm_gate(const at::Tensor& o, const at::Tensor& w, const at::Tensor& g, double eps, bool out_bf16) {
+at::Tensor headnorm_gate(const at::Tensor& o, const at::Tensor& w, const at::Tensor& g, double eps, bool out_bf16, bool silu) {
   HYB_CHECK(o.is_cuda() && o.is_contiguous() && o.dim() == 3 && o.scalar_type() == at::kFloat, "o: contiguous fp32 [T, H, dv]");
   check_rows(g, "g");
   const int64_t T = o.size(0);
@@ -372,7 +374,7 @@ at::Tensor headnorm_gate(const at::Tensor& o, const at::Tensor& w, const at::Ten
   dispatch_act(g, [&](auto* tag) {
     using Tt = std::remove_pointer_t<decltype(tag)>;
     headnorm_gate_kernel<Tt><<<dim3((unsigned)((pairs + NW - 1) / NW)), NT, 0, cur_stream()>>>(
-        o.data_ptr<float>(), w.data_ptr<float>(), (const Tt*)g.data_ptr(), g.stride(0), (Tt*)y.data_ptr(), pairs, H, dv, (float)eps);
+        o.data_ptr<float>(), w.data_ptr<float>(), (const Tt*)g.data_ptr(), g.stride(0), (Tt*)y.data_ptr(), pairs, H, dv, (float)eps, silu ? 1 : 0);
   });
   return y;
 }
