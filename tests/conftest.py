@@ -9,7 +9,7 @@ if ROOT not in sys.path:
 
 
 def pytest_configure(config):
-    config.addinivalue_line("markers", "gpu: needs an MI355X (runs via gpurun on the GPU box)")
+    config.addinivalue_line("markers", "gpu: needs an MI355X")
     config.addinivalue_line("markers", "multigpu: needs >=2 GPUs")
     config.addinivalue_line("markers", "slow: long-running test")
 
