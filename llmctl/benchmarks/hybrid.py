@@ -1,7 +1,9 @@
 """Serving throughput of a Lenitar configuration beside the closest existing model (the routed-expert
 transformer: softmax attention + top-k SwiGLU experts) at equal width, depth, heads and experts, and of
 a Dumalix configuration beside the dense transformer (grouped-query softmax attention + SwiGLU) at equal
-width, layer runs, heads, kv heads and feed-forward size.
+width, layer runs, heads, kv heads and feed-forward size, and of a Malinex configuration beside Lenitar (the
+closest existing model: recurrent-state layers among attention layers, routed experts, an fp32 residual
+stream) at equal width, depth, heads, experts and expert size.
 
 Both run through the same engine calls: one prompt portion per sequence (``InferenceEngine.prefill``)
 and then one-token decode steps of the whole batch (``InferenceEngine.decode``); random weights,
@@ -33,6 +35,28 @@ DUMALIX_SIZES = {
     "medium": dict(width=2048, layers=6, loop=(2, 5, 2), heads=16, kv_heads=4, head_dim=128, ff=6144, chunk=1024, prompt=2048, batch=16),
     "large": dict(width=4096, layers=6, loop=(2, 5, 2), heads=32, kv_heads=8, head_dim=128, ff=12288, chunk=2048, prompt=4096, batch=16),
 }
+
+
+# Malinex: width, layers (every third is sigmoid attention, the others gated linear attention), heads of
+# ``head_dim`` (gated linear attention: keys of half that), kv heads, routed experts + one shared, prompt, decode batch
+MALINEX_SIZES = {
+    "tiny": dict(width=128, layers=3, heads=4, kv_heads=2, head_dim=32, experts=4, top=2, ff=64, prompt=64, batch=2),
+    "small": dict(width=1024, layers=6, heads=8, kv_heads=2, head_dim=128, experts=8, top=2, ff=512, prompt=2048, batch=16),
+    "medium": dict(width=2048, layers=6, heads=16, kv_heads=4, head_dim=128, experts=8, top=2, ff=1024, prompt=2048, batch=16),
+}  # (no width 4096: Lenitar's latent rank of width / 4 is then beyond its attention kernels)
+
+
+def _configs_malinex(s: Dict):
+    from llmctl.models.lenitar import lenitar_template
+    from llmctl.models.malinex import malinex_template
+
+    ma = malinex_template(width=s["width"], layers=s["layers"], heads=s["heads"], kv_heads=s["kv_heads"], vocab=32000, every=3,
+                          experts=s["experts"], top=s["top"], expert_ff=s["ff"], head_dim=s["head_dim"],
+                          max_positions=s["prompt"] + 256)
+    le = lenitar_template(width=s["width"], layers=s["layers"], heads=s["heads"], vocab=32000, every=3, experts=s["experts"],
+                          top=s["top"], groups=2, keep=1, ff=s["ff"], window=s["prompt"])
+    le.max_position_embeddings = s["prompt"] + 256
+    return ma, le
 
 
 def _configs_dumalix(s: Dict):
@@ -127,7 +151,12 @@ def _measure(eng, prompt: int, batch: int, steps: int, warmup: int) -> Dict[str,
 def run(sizes: List[str], device: str = "auto", steps: int = 5, warmup: int = 2, family: str = "lenitar") -> List[Dict]:
     out = []
     for name in sizes:
-        if family == "dumalix":
+        if family == "malinex":
+            s = MALINEX_SIZES[name]
+            hy, tr = _configs_malinex(s)
+            row = {"size": name, **s}
+            pair = (("malinex", hy), ("lenitar", tr))
+        elif family == "dumalix":
             s = DUMALIX_SIZES[name]
             hy, tr = _configs_dumalix(s)
             row = {"size": name, **s, "layer_runs": len(hy.runs())}
