@@ -240,7 +240,10 @@ class BiasedSoftmaxMoE(nn.Module):
     few tokens that between them reach about every expert anyway (decode batches) take the dense form
     instead: all experts on all rows in one up GEMM, one activation pass and one batched down GEMM on the
     stacked weights, the unchosen experts weighted by zero; that form has no host synchronisation and a
-    quarter of the launches.  The shared expert's up projection carries ``side`` extra output rows (with a
+    quarter of the launches.  Longer steps run one pair of GEMMs per expert.  (A third form, all experts as one
+    batch of equal-sized segments through two batched GEMMs on the stacked weights, is written and agrees with
+    the others on the CPU and on small GPU steps, but a 2048-token step through it ended in a GPU memory fault
+    whose cause is not found: ``BATCHED`` keeps it off on GPUs.)  The shared expert's up projection carries ``side`` extra output rows (with a
     bias) that are handed back; without a shared expert they are a projection of their own."""
 
     def __init__(self, width: int, ff: int, experts: int, top: int, act: str = "relu2", shared_ff: int = 0,
@@ -278,6 +281,34 @@ class BiasedSoftmaxMoE(nn.Module):
     def _dense(self, T: int) -> bool:
         return T <= self.DENSE_ROWS and T * self.top >= self.E
 
+    BATCHED = False  # the batched-segment form on GPUs: off (see the class docstring)
+
+    def _batched(self, N: int, C: int) -> bool:
+        """N token copies in segments padded to C rows each: worth it unless the padding doubles the work."""
+        return (self.BATCHED or not self.w_up.is_cuda) and self.E * C <= 2 * N + self.E * self.PAD
+
+    def _run_batched(self, xs: torch.Tensor, counts: List[int], C: int, act) -> torch.Tensor:
+        """``xs``: the token copies sorted by expert, zero rows from row N on.  Gathers every expert's segment
+        into ``[E, C, width]`` (missing rows = the zero row N), runs both projections as batched GEMMs and
+        gathers the N real rows back in sorted order."""
+        import numpy as np
+
+        E, N, W = self.E, sum(counts), xs.shape[1]
+        gi = np.full(E * C, N, dtype=np.int64)
+        back = np.empty(N, dtype=np.int64)
+        o = 0
+        for e, n in enumerate(counts):
+            gi[e * C:e * C + n] = np.arange(o, o + n)
+            back[o:o + n] = np.arange(e * C, e * C + n)
+            o += n
+        # a blocking copy: the host array is a temporary, and an asynchronous copy from pageable memory of this
+        # size may read it after it has been released
+        both = torch.from_numpy(np.concatenate([gi, back])).to(xs.device)
+        xg = xs.index_select(0, both[:E * C]).view(E, C, W)
+        a = act(torch.bmm(xg, self.w_up.transpose(1, 2)).view(E * C, self.ff))
+        y = torch.bmm(a.view(E, C, self.ff), self.w_down.transpose(1, 2)).view(E * C, W)
+        return y.index_select(0, both[E * C:])
+
     def forward(self, x: torch.Tensor):
         """x [T, width] -> fp32 [T, width] (and the side columns)."""
         from llmctl.ops import hybrid as hops
@@ -298,7 +329,12 @@ class BiasedSoftmaxMoE(nn.Module):
             tok = torch.div(order, self.top, rounding_mode="floor")
             xs = x.new_zeros((tok.shape[0] + self.PAD, x.shape[1]))  # spare rows: see run_expert_segments
             torch.index_select(x, 0, tok, out=xs[:tok.shape[0]])
-            ye = run_expert_segments(xs, counts, self.experts_up, self.experts_down, act, pad=self.PAD)
+            big = max(counts)
+            C = 16 if big <= 16 else (big + self.PAD - 1) // self.PAD * self.PAD
+            if self._batched(tok.shape[0], C):
+                ye = self._run_batched(xs, counts, C, act)
+            else:
+                ye = run_expert_segments(xs, counts, self.experts_up, self.experts_down, act, pad=self.PAD)
             w = topw.reshape(-1).index_select(0, order).unsqueeze(-1)
             out = torch.zeros(T, x.shape[1], dtype=torch.float32, device=x.device).index_add_(0, tok, ye.float() * w)
         side = None

@@ -283,7 +283,7 @@ def gla_chunk_plan(cu_host, device):
             pcu.append(t)
         base.append(len(pcu) - 1)
     P = len(pcu) - 1
-    both = torch.tensor(pcu + base, dtype=torch.int32).to(device, non_blocking=True)
+    both = torch.tensor(pcu + base, dtype=torch.int32).to(device)  # blocking: the host tensor is a temporary
     ident = torch.arange(P, dtype=torch.int32, device=device)
     return (both[:P + 1], both[P + 1:], ident, torch.zeros(P, dtype=torch.int32, device=device),
             torch.ones(P, dtype=torch.int32, device=device), P)

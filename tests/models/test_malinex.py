@@ -143,13 +143,18 @@ def test_routed_feed_forward(tmp_path, dev, f):
     check(tmp_path, dev, cfg, r, whole(r), bf16_tol=0.25)
 
 
-@pytest.mark.parametrize("dense", [False, True])
-def test_routed_and_dense_expert_forms(tmp_path, dev, dense, monkeypatch):
-    # steps of few rows run all experts on all rows (unchosen ones weighted by zero), longer ones sort token copies
-    # into per-expert segments; here every step is forced into one form
+@pytest.mark.parametrize("form", ["dense", "batched", "segments"])
+def test_expert_forms(tmp_path, dev, form, monkeypatch):
+    # steps of few rows run all experts on all rows (unchosen ones weighted by zero); longer ones sort token copies by
+    # expert and run the segments as one batch padded to the largest, or, if routing is unbalanced, one by one;
+    # here every step is forced into one form
     from llmctl.models.moe import BiasedSoftmaxMoE
 
-    monkeypatch.setattr(BiasedSoftmaxMoE, "_dense", lambda self, T: dense)
+    if form == "batched" and dev[0] == "cuda":
+        pytest.skip("the batched-segment form is switched off on GPUs: a 2048-token step through it ended in a GPU "
+                    "memory fault whose cause is not found")
+    monkeypatch.setattr(BiasedSoftmaxMoE, "_dense", lambda self, T: form == "dense")
+    monkeypatch.setattr(BiasedSoftmaxMoE, "_batched", lambda self, N, C: form == "batched")
     cfg = U.config([(U.gla(), U.moe(experts=7, top=3, ff=9, shared=5)), (U.att(), U.moe(experts=3, top=1, ff=16, shared=0))])
     r = {"a": tokens(70, 50, 40), "b": tokens(6, 50, 41)}
     check(tmp_path, dev, cfg, r, [[("a", 1)], [("a", 66), ("b", 2)], [("a", 3), ("b", 4)]], bf16_tol=0.25)
