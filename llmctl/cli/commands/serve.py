@@ -42,7 +42,7 @@ def start(
     p = Path(artifact)
     from llmctl.models.config import ALIASES
 
-    if not p.exists() and artifact.lower() not in ALIASES and not artifact.lower().startswith(("lenitar-", "dumalix-", "malinex-")):
+    if not p.exists() and artifact.lower() not in ALIASES and not artifact.lower().startswith(("lenitar-", "dumalix-", "malinex-", "pamazen-")):
         console.print(f"[red]Artifact not found: {artifact}[/red]")
         raise typer.Exit(1)
     console.print("[blue]Starting inference server...[/blue]")

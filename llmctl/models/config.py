@@ -292,6 +292,12 @@ def get_model_config(name_or_path: str) -> ModelConfig:
         kv = {p[0]: int(p[1:]) for p in key.split("-")[1:] if p[1:].isdigit()}
         return malinex_template(width=kv.get("w", 256), layers=kv.get("l", 4), heads=kv.get("h", 4),
                                 kv_heads=kv.get("g", 2), experts=kv.get("e", 0), share=bool(kv.get("s", 0)))
+    if key.startswith("pamazen-"):  # pamazen-w<width>-l<layers>[-h<heads>][-g<kv heads>][-e<experts>][-s<streams>]: random-init template
+        from .pamazen import pamazen_template
+
+        kv = {p[0]: int(p[1:]) for p in key.split("-")[1:] if p[1:].isdigit()}
+        return pamazen_template(width=kv.get("w", 256), layers=kv.get("l", 4), heads=kv.get("h", 4),
+                                kv_heads=kv.get("g", 2), experts=kv.get("e", 8), streams=kv.get("s", 4))
     if key in ALIASES:
         t, s = ALIASES[key]
         return ModelConfig.from_dict(MODEL_TEMPLATES[t][s])

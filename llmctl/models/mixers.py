@@ -76,11 +76,14 @@ def rotary_frequencies(base: float, dims: int, scaling: Optional[dict] = None, d
     ``scaling`` = ``{factor, original, fast, slow}`` applies YaRN: with ``where(t) = dims ln(original /
     (2 pi t)) / (2 ln base)`` the pairs below ``floor(where(fast))`` keep their frequency, those above
     ``ceil(where(slow))`` are divided by ``factor``, a linear ramp lies between; cos and sin are multiplied
-    by ``0.1 ln(factor) + 1``."""
+    by ``0.1 ln(factor) + 1``.  ``scaling`` = ``{factor}`` alone is linear scaling: every frequency is divided
+    by ``factor``."""
     i = torch.arange(dims // 2, dtype=torch.float64)
-    f = float(base) ** (-2.0 * i / dims)
+    f = float(base) ** (-2.0 * i / max(dims, 1))
     amp = 1.0
-    if scaling:
+    if scaling and "original" not in scaling:
+        f = f / float(scaling.get("factor", 1.0))
+    elif scaling:
         factor, orig = float(scaling["factor"]), float(scaling["original"])
         where = lambda t: dims * math.log(orig / (2.0 * math.pi * t)) / (2.0 * math.log(float(base)))
         lo = max(math.floor(where(float(scaling["fast"]))), 0)
@@ -231,37 +234,57 @@ class CausalConv(nn.Module):
 class GroupedAttention(nn.Module):
     """Grouped-query attention (``heads`` query heads over ``kv_heads`` key / value heads; key size
     ``dim``, value size ``vdim``) with, each optional: ``conv_taps`` short causal convolutions on the
-    projected q, k, v; per-head RMS norm of q and k; rotary on the first ``rot_dims`` entries (YaRN by
-    ``rot_scaling``, neighbour pairs when ``interleaved``); ``rotate_values``: the value of position j
+    projected q, k, v; ``qk_norm``: per-head RMS norm of q and k; rotary on the first ``rot_dims`` entries (YaRN
+    or linear scaling by ``rot_scaling``, neighbour pairs when ``interleaved``); ``rotate_values``: the value of position j
     is cached turned by ``j * rot_base^(-2m/vdim)`` per pair m and a head's output at position i is
     turned back by i, so the sum weighs values by their relative position; ``temperature``: a learned
-    per-head factor on the scaled scores; ``chunk``: position i sees j <= i of its own chunk of that
-    many positions only; ``window``; ``sink``: a learned per-head logit that joins the softmax
-    denominator (not scaled, no value).  The cache row of a token is ``[v | k]`` per kv head."""
+    per-head factor on the scaled scores; ``softcap`` c: the scaled score becomes ``c tanh(score / c)``;
+    ``chunk``: position i sees j <= i of its own chunk of that many positions only; ``window``, of which
+    ``keep_first`` exempts the first positions of the sequence; ``sink``: True = a learned per-head logit that
+    joins the softmax denominator (not scaled, not capped, no value), a number = that logit fixed for all heads
+    (0.0: one is added to the denominator).  ``values="keys"``: there is no value projection; a token's value is
+    the output of its key projection, taken ahead of norm and rotary.  ``value_mix``: ``"source"`` leaves the step's projected values
+    where a later layer finds them, ``"mix"`` replaces v by ``(1 - vmix) v + vmix v_source`` (same token, one learned
+    number) before it is cached.  The cache row of a token is ``[v | k]`` per kv head."""
 
     def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, rot_base: float, rot_dims: int,
                  scale: float, eps: float, conv_taps: int = 0, rot_scaling: Optional[dict] = None,
                  interleaved: bool = True, rotate_values: bool = False, temperature: bool = False,
-                 chunk: Optional[int] = None, window: Optional[int] = None, sink: bool = False, device=None, dtype=None):
+                 chunk: Optional[int] = None, window: Optional[int] = None, sink=False, qk_norm: bool = True,
+                 values: str = "own", value_mix: Optional[str] = None, softcap: float = 0.0, keep_first: int = 0,
+                 device=None, dtype=None):
         super().__init__()
         if heads % kv_heads or rot_dims % 2 or rot_dims > dim:
             raise ValueError("kv heads must divide the heads; rotary dims must be even and fit the head")
         if rotate_values and (vdim % 2 or not interleaved):
             raise ValueError("turned values need an even value size and neighbour pairs")
+        if values not in ("own", "keys") or (values == "keys" and (vdim != dim or rotate_values or value_mix or conv_taps)):
+            raise ValueError("values that are the keys have the keys' size and are neither turned, mixed nor convolved")
+        if value_mix not in (None, "source", "mix"):
+            raise ValueError("value_mix: None, 'source' or 'mix'")
         self.width, self.H, self.G, self.dk, self.dv = width, heads, kv_heads, dim, vdim
         self.rot_dims, self.scale, self.eps, self.interleaved = rot_dims, scale, eps, interleaved
         self.chunk = int(chunk) if chunk else hops.NO_LIMIT
         self.window = int(window) if window else hops.NO_LIMIT
+        self.softcap, self.keep_first = float(softcap or 0.0), int(keep_first or 0)
+        self.v_from_k, self.value_mix = values == "keys", value_mix
         kw = dict(device=device, dtype=dtype)
         f32 = dict(device=device, dtype=torch.float32)
-        cols = (heads + kv_heads) * dim + kv_heads * vdim
+        cols = (heads + kv_heads) * dim + (0 if self.v_from_k else kv_heads * vdim)
+        self.cols = cols
         self.w_qkv = nn.Parameter(torch.empty(cols, width, **kw))  # [W_q ; W_k ; W_v]: the input is read once
         self.w_o = nn.Parameter(torch.empty(width, heads * vdim, **kw))
         self.conv = CausalConv(cols, conv_taps, residual=False, device=device) if conv_taps else None
-        self.q_norm = nn.Parameter(torch.ones(dim, **f32))
-        self.k_norm = nn.Parameter(torch.ones(dim, **f32))
+        self.q_norm = nn.Parameter(torch.ones(dim, **f32)) if qk_norm else None
+        self.k_norm = nn.Parameter(torch.ones(dim, **f32)) if qk_norm else None
         self.temp = nn.Parameter(torch.ones(heads, **f32)) if temperature else None
-        self.sink = nn.Parameter(torch.zeros(heads, **f32)) if sink else None
+        if sink is True:
+            self.sink = nn.Parameter(torch.zeros(heads, **f32))
+        elif sink is False or sink is None:
+            self.sink = None
+        else:
+            self.register_buffer("sink", torch.full((heads,), float(sink), **f32), persistent=False)
+        self.vmix = nn.Parameter(torch.zeros(1, **f32)) if value_mix else None
         for w in (self.w_qkv, self.w_o):
             _init(w, 0.02)
         inv_freq, self.rot_amp = rotary_frequencies(rot_base, rot_dims, rot_scaling, device)
@@ -270,23 +293,39 @@ class GroupedAttention(nn.Module):
         self.register_buffer("v_freq", vf, persistent=False)
 
     cache_kind = "latent"  # a paged pool of rows
+    VALUE_SOURCE = "values_of_first_mixing_layer"  # key in StepBatch.scratch
 
     @property
     def cache_row(self) -> int:
         return self.G * (self.dv + self.dk)
 
+    @property
+    def w_in(self):
+        return self.w_qkv
+
     def state_shapes(self):
         return [self.conv.state_shape()] if self.conv is not None else []
 
-    def step(self, h: torch.Tensor, b: StepBatch, cache) -> torch.Tensor:
-        rows, states = cache
+    def step(self, h: torch.Tensor, b: StepBatch, cache, z: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``z``: the input projection ``h W_qkv^T`` if the caller has made it (as columns of a wider product)."""
+        rows, states = cache if isinstance(cache, tuple) else (cache, ())
         T = h.shape[0]
-        z = F.linear(h, self.w_qkv)
+        if z is None:
+            z = F.linear(h, self.w_qkv)
         if self.conv is not None:
             z = self.conv(z, b, states[0])
+        v_first = None
+        if self.value_mix is not None:
+            v0 = (self.H + self.G) * self.dk
+            if self.value_mix == "source":
+                b.scratch[self.VALUE_SOURCE] = z[:, v0:v0 + self.G * self.dv]
+            else:
+                v_first = b.scratch[self.VALUE_SOURCE]
         q = hops.attn_qkv_prep(z, self.H, self.G, self.dk, self.dv, self.q_norm, self.k_norm, self.eps, b.pos,
-                               self.inv_freq, self.rot_dims, self.interleaved, self.rot_amp, self.v_freq, rows, b.slots)
-        opt = dict(groups=self.G, koff=self.dv, chunk=self.chunk, hscale=self.temp, ofreq=self.v_freq)
+                               self.inv_freq, self.rot_dims, self.interleaved, self.rot_amp, self.v_freq, rows, b.slots,
+                               v_from_k=self.v_from_k, v_first=v_first, v_lambda=self.vmix if v_first is not None else None)
+        opt = dict(groups=self.G, koff=self.dv, chunk=self.chunk, hscale=self.temp, ofreq=self.v_freq,
+                   softcap=self.softcap, keep_first=self.keep_first)
         outs = []
         if b.Tp:
             outs.append(hops.latent_attention_prefill(q[:b.Tp], rows, b.p_bt, b.p_cu, b.p_ctx, self.window, self.sink,
@@ -494,3 +533,94 @@ class DenseFF(nn.Module):
         z = F.linear(h, self.w_up, self.b_up)
         y = F.linear(hops.act_any(z[:, :self.ff], self.act), self.w_down)
         return (y, z[:, self.ff:]) if self.side else y
+
+
+class DeltaRule(nn.Module):
+    """The generalized delta rule: per head a memory ``S [dim, dim]`` with ``S_t = diag(w_t) S_(t-1) - (a_t u_t)
+    (u_t^T S_(t-1)) + k_t v_t^T`` (both terms read the old memory) and ``o_t = S_t^T r_t``, where ``r, k, v = W_r h,
+    W_k h, W_v h``, the decay per key channel is ``w = exp(-decay_coef sigmoid(W_w2 tanh(W_w1 h) + w0))``, the removal
+    rate ``a = sigmoid(W_a h + b_a)`` and ``u = k / sqrt(sum k^2 + key_eps)`` the unit key of the head.  Each head's
+    ``o`` is divided by its root mean square, the heads are concatenated, multiplied by the weight ``norm`` and by
+    ``sigmoid(W_g h)``, then projected by ``W_o``.  The memory is fp32 and lives in a state slot per sequence.
+    The fused input weight is ``[W_r ; W_k ; W_v ; W_g ; W_a ; W_w1]``."""
+
+    def __init__(self, width: int, heads: int, dim: int, decay_rank: int, eps: float, decay_coef: float = math.exp(-0.5),
+                 key_eps: float = 1e-6, device=None, dtype=None):
+        super().__init__()
+        self.width, self.H, self.d, self.rank, self.eps = width, heads, dim, decay_rank, eps
+        self.decay_coef, self.key_eps = float(decay_coef), float(key_eps)
+        kw = dict(device=device, dtype=dtype)
+        f32 = dict(device=device, dtype=torch.float32)
+        n = heads * dim
+        self.cols = 5 * n + decay_rank
+        self.w_in = nn.Parameter(torch.empty(self.cols, width, **kw))
+        self.w_w2 = nn.Parameter(torch.empty(n, decay_rank, **kw))
+        self.w0 = nn.Parameter(torch.zeros(n, **f32))
+        self.b_a = nn.Parameter(torch.zeros(n, **f32))
+        self.norm = nn.Parameter(torch.ones(n, **f32))
+        self.w_o = nn.Parameter(torch.empty(width, n, **kw))
+        for w in (self.w_in, self.w_w2, self.w_o):
+            _init(w, 0.02)
+
+    cache_kind = "state"
+    cache_row = 0
+
+    def state_shapes(self):
+        return [(self.H, self.d, self.d)]
+
+    def step(self, h: torch.Tensor, b: StepBatch, state, z: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if isinstance(state, tuple) and len(state) == 2 and isinstance(state[1], tuple):  # (rows, states)
+            state = state[1]
+        T, H, d = h.shape[0], self.H, self.d
+        n = H * d
+        if z is None:
+            z = F.linear(h, self.w_in)
+        r, k, v = (z[:, i * n:(i + 1) * n].unflatten(1, (H, d)) for i in range(3))
+        g, za = z[:, 3 * n:4 * n], z[:, 4 * n:5 * n]
+        zw = _mm_f32(hops.tanh_act(z[:, 5 * n:self.cols]), self.w_w2)  # fp32 [T, H * d]
+        if "gla_plan" not in b.scratch:
+            b.scratch["gla_plan"] = hops.gla_chunk_plan(b.cu_host, h.device) if h.is_cuda else None
+        o = hops.delta_scan(r, k, v, zw, self.w0, za, self.b_a, self.decay_coef, self.key_eps, state[0], b.state, b.cu,
+                            b.start, plan=b.scratch["gla_plan"])
+        return F.linear(hops.headnorm_gate(o, self.norm, g, self.eps, h.dtype), self.w_o)
+
+
+class ParallelMixers(nn.Module):
+    """Two mixers side by side on the same input: the result is ``left_scale * left(h) + right_scale * right(h)``.
+    ``step`` returns the two results with their factors (the layer's residual pass sums them); both input
+    projections run as one product on the stacked weights, so the input is read once.  The cache entry is the
+    pair the members need: paged rows for the one that attends, state pools for the one that recurs."""
+
+    def __init__(self, left: nn.Module, right: nn.Module, left_scale: float, right_scale: float):
+        super().__init__()
+        self.left, self.right = left, right
+        self.left_scale, self.right_scale = float(left_scale), float(right_scale)
+        self._w, self._w_key = None, None
+
+    @property
+    def cache_kind(self):
+        return "rows+state"
+
+    @property
+    def cache_row(self) -> int:
+        return int(self.left.cache_row) + int(self.right.cache_row)
+
+    def state_shapes(self):
+        return list(self.left.state_shapes()) + list(self.right.state_shapes())
+
+    def _stacked(self) -> torch.Tensor:
+        """[W_in left ; W_in right] (made once; serving weights are static)."""
+        a, c = self.left.w_in, self.right.w_in
+        key = (a.data_ptr(), a._version, c.data_ptr(), c._version)
+        if self._w_key != key:
+            self._w, self._w_key = torch.cat([a.detach(), c.detach()], 0).contiguous(), key
+        return self._w
+
+    def step(self, h: torch.Tensor, b: StepBatch, cache):
+        rows, states = cache
+        nl = len(self.left.state_shapes())
+        z = F.linear(h, self._stacked())
+        cl = self.left.w_in.shape[0]
+        yl = self.left.step(h, b, (rows, tuple(states[:nl])), z=z[:, :cl])
+        yr = self.right.step(h, b, (rows, tuple(states[nl:])), z=z[:, cl:])
+        return (yl, self.left_scale), (yr, self.right_scale)

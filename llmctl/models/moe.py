@@ -232,10 +232,16 @@ class GroupLimitedMoE(nn.Module):
 
 
 class BiasedSoftmaxMoE(nn.Module):
-    """Routed ungated experts ``W_down act(W_up h)`` chosen by softmax scores plus a selection bias
-    (serving forward).  Router logits are an fp32 product; ``s = softmax(z)``; the ``top`` experts with the
-    largest ``s + bias`` are used, weighted by their own ``s`` over the sum of the chosen ones; an
-    optional shared expert of the same form runs for every token.  Dispatch as in :class:`GroupLimitedMoE`
+    """Routed experts chosen by softmax scores plus a selection bias (serving forward).  Router logits are an
+    fp32 product; ``s = softmax(z)``; the ``top`` experts with the largest ``s + bias`` are used, weighted by their
+    own ``s`` (over the sum of the chosen ones when ``renorm``); an optional shared expert of the same form runs
+    for every token.  Experts: ``W_down act(W_up h)`` with ``act`` = ``relu2`` / ``gelu``, or gated, ``W_down
+    (silu(W_gate h) * W_up h)``, with ``act="swiglu"`` (gate and up are one weight ``[gate ; up]``).  Options:
+    ``groups`` / ``keep``: the router's outputs form equal groups of neighbours, a group scores as its best choice
+    score, and only experts of the ``keep`` best groups can be chosen; ``identity``: the last that many router
+    outputs are experts without weights whose output is their input; ``shared_gate``: the shared expert's output is
+    multiplied by ``sigmoid(w_sg . h)``, one number per token, whose row rides on the shared up projection.
+    Dispatch as in :class:`GroupLimitedMoE`
     (token copies sorted by expert, per-expert GEMMs on contiguous segments, fp32 weighted sum).  Steps of
     few tokens that between them reach about every expert anyway (decode batches) take the dense form
     instead: all experts on all rows in one up GEMM, one activation pass and one batched down GEMM on the
@@ -247,19 +253,29 @@ class BiasedSoftmaxMoE(nn.Module):
     bias) that are handed back; without a shared expert they are a projection of their own."""
 
     def __init__(self, width: int, ff: int, experts: int, top: int, act: str = "relu2", shared_ff: int = 0,
-                 side: int = 0, device=None, dtype=None):
+                 side: int = 0, groups: int = 1, keep: int = 1, renorm: bool = True, identity: int = 0,
+                 shared_gate: bool = False, device=None, dtype=None):
         super().__init__()
-        if not (0 < top <= experts):
+        n = experts + identity
+        if not (0 < top <= n):
             raise ValueError("router: top must lie in 1 .. experts")
+        if groups < 1 or n % groups or not (0 < keep <= groups) or top > keep * (n // groups):
+            raise ValueError("router: its outputs must split into equal groups and top must fit the kept groups")
+        if shared_gate and not shared_ff:
+            raise ValueError("a gate on the shared expert needs a shared expert")
         self.E, self.top, self.ff, self.act, self.shared_ff, self.side = experts, top, ff, act, shared_ff, side
+        self.groups, self.keep, self.renorm, self.identity, self.shared_gate = groups, keep, renorm, identity, shared_gate
+        self.up_rows = 2 * ff if act == "swiglu" else ff  # rows of an expert's first projection
+        self.sup_rows = 2 * shared_ff if act == "swiglu" else shared_ff
+        extra = self.sup_rows + (1 if shared_gate else 0) + side
         kw = dict(device=device, dtype=dtype)
         f32 = dict(device=device, dtype=torch.float32)
-        self.w_router = nn.Parameter(torch.empty(experts, width, **f32))
-        self.bias = nn.Parameter(torch.zeros(experts, **f32))
-        self.w_up = nn.Parameter(torch.empty(experts, ff, width, **kw))  # stacked: expert e is w_up[e]
+        self.w_router = nn.Parameter(torch.empty(n, width, **f32))
+        self.bias = nn.Parameter(torch.zeros(n, **f32))
+        self.w_up = nn.Parameter(torch.empty(experts, self.up_rows, width, **kw))  # stacked: expert e is w_up[e]
         self.w_down = nn.Parameter(torch.empty(experts, width, ff, **kw))
-        self.w_sup = nn.Parameter(torch.empty(shared_ff + side, width, **kw)) if shared_ff + side else None
-        self.b_sup = nn.Parameter(torch.zeros(shared_ff + side, **kw)) if side else None
+        self.w_sup = nn.Parameter(torch.empty(extra, width, **kw)) if extra else None
+        self.b_sup = nn.Parameter(torch.zeros(extra, **kw)) if side else None
         self.w_sdown = nn.Parameter(torch.empty(width, shared_ff, **kw)) if shared_ff else None
         with torch.no_grad():
             self.w_router.normal_(0.0, 0.02)
@@ -305,7 +321,7 @@ class BiasedSoftmaxMoE(nn.Module):
         # size may read it after it has been released
         both = torch.from_numpy(np.concatenate([gi, back])).to(xs.device)
         xg = xs.index_select(0, both[:E * C]).view(E, C, W)
-        a = act(torch.bmm(xg, self.w_up.transpose(1, 2)).view(E * C, self.ff))
+        a = act(torch.bmm(xg, self.w_up.transpose(1, 2)).view(E * C, self.up_rows))
         y = torch.bmm(a.view(E, C, self.ff), self.w_down.transpose(1, 2)).view(E * C, W)
         return y.index_select(0, both[E * C:])
 
@@ -314,35 +330,45 @@ class BiasedSoftmaxMoE(nn.Module):
         from llmctl.ops import hybrid as hops
 
         T = x.shape[0]
-        act = lambda u: hops.act_any(u, self.act)
-        topi, topw = hops.bias_topk_router(torch.nn.functional.linear(x.float(), self.w_router), self.bias, self.top)
+        act = hops.swiglu_any if self.act == "swiglu" else (lambda u: hops.act_any(u, self.act))
+        topi, topw = hops.bias_topk_router(torch.nn.functional.linear(x.float(), self.w_router), self.bias, self.top,
+                                           self.groups, self.keep, self.renorm)
         if self._dense(T):
             E, ff, W = self.E, self.ff, x.shape[1]
-            a = act(torch.nn.functional.linear(x, self.w_up.view(E * ff, W)))  # [T, E * ff]
+            a = act(torch.nn.functional.linear(x, self.w_up.view(E * self.up_rows, W)).view(T * E, self.up_rows))  # [T * E, ff]
             y = torch.bmm(a.view(T, E, ff).transpose(0, 1), self.w_down.transpose(1, 2))  # [E, T, W]
-            dw = torch.zeros(T, E, dtype=torch.float32, device=x.device).scatter_(1, topi, topw)
-            out = (y.float() * dw.t().unsqueeze(-1)).sum(0)
+            dw = torch.zeros(T, E + self.identity, dtype=torch.float32, device=x.device).scatter_(1, topi, topw)
+            out = (y.float() * dw[:, :E].t().unsqueeze(-1)).sum(0)
+            if self.identity:
+                out += x.float() * dw[:, E:].sum(1, keepdim=True)
         else:
             flat = topi.reshape(-1)
-            counts = torch.bincount(flat, minlength=self.E).tolist()  # the layer's one host sync
+            counts = torch.bincount(flat, minlength=self.E + self.identity).tolist()  # the layer's one host sync
             order = torch.argsort(flat, stable=True)
             tok = torch.div(order, self.top, rounding_mode="floor")
             xs = x.new_zeros((tok.shape[0] + self.PAD, x.shape[1]))  # spare rows: see run_expert_segments
             torch.index_select(x, 0, tok, out=xs[:tok.shape[0]])
-            big = max(counts)
+            real = sum(counts[:self.E])  # copies that go to experts with weights; the identity experts' follow
+            big = max(counts[:self.E]) if self.E else 0
             C = 16 if big <= 16 else (big + self.PAD - 1) // self.PAD * self.PAD
-            if self._batched(tok.shape[0], C):
+            if not self.identity and self._batched(tok.shape[0], C):
                 ye = self._run_batched(xs, counts, C, act)
             else:
-                ye = run_expert_segments(xs, counts, self.experts_up, self.experts_down, act, pad=self.PAD)
+                ye = run_expert_segments(xs, counts[:self.E], self.experts_up, self.experts_down, act, pad=self.PAD)
+                if real < tok.shape[0]:
+                    ye = torch.cat([ye, xs[real:tok.shape[0]]], 0)
             w = topw.reshape(-1).index_select(0, order).unsqueeze(-1)
             out = torch.zeros(T, x.shape[1], dtype=torch.float32, device=x.device).index_add_(0, tok, ye.float() * w)
         side = None
         if self.w_sup is not None:
             z = torch.nn.functional.linear(x, self.w_sup, self.b_sup)
             if self.shared_ff:
-                out += torch.nn.functional.linear(act(z[:, :self.shared_ff]), self.w_sdown)
-            side = z[:, self.shared_ff:]
+                ys = torch.nn.functional.linear(act(z[:, :self.sup_rows]), self.w_sdown)
+                if self.shared_gate:
+                    out = hops.gated_add_f32_(out, ys, z[:, self.sup_rows:self.sup_rows + 1])
+                else:
+                    out += ys
+            side = z[:, self.sup_rows + (1 if self.shared_gate else 0):]
         return (out, side) if self.side else out
 
 

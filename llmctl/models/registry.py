@@ -63,5 +63,14 @@ def _register_builtin() -> None:
 
     register(malinex.ARCHITECTURE, Family(malinex.MalinexConfig, build_malinex, malinex.load_malinex))
 
+    from . import pamazen
+
+    def build_pamazen(cfg, device=None, dtype=torch.bfloat16, seed=None):
+        if seed is not None:
+            torch.manual_seed(seed)
+        return pamazen.PamazenLM(cfg, device=device, dtype=dtype)
+
+    register(pamazen.ARCHITECTURE, Family(pamazen.PamazenConfig, build_pamazen, pamazen.load_pamazen))
+
 
 _register_builtin()

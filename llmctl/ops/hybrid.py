@@ -76,7 +76,7 @@ NO_LIMIT = 1 << 30  # a window or chunk that never masks
 
 def latent_attention_prefill(qa, cache, bt, cu, ctx, window: int, sink, scale: float, rk: int, max_q: int,
                              mfma: bool = True, groups: int = 1, koff: int = 0, chunk: int = NO_LIMIT, hscale=None,
-                             ofreq=None, sig_bias=None, dist_a=None, dist_b=None):
+                             ofreq=None, sig_bias=None, dist_a=None, dist_b=None, softcap: float = 0.0, keep_first: int = 0):
     """Prompt portions: sequence n's query rows ``[cu[n], cu[n+1])`` end at position ``ctx[n]-1``;
     ``max_q``: the longest portion (sizes the launch).  bf16 shapes that fit run on the matrix cores
     (``mfma=False`` forces the generic fp32-SIMT kernel, which also serves fp32).
@@ -89,25 +89,28 @@ def latent_attention_prefill(qa, cache, bt, cu, ctx, window: int, sink, scale: f
     scores; ``ofreq`` (fp32 [rk/2]) turns the output's neighbour pairs back by ``-position * ofreq``.
     ``dist_a``, ``dist_b`` (fp32 [H], together): ``dist_a ln(1 + dist_b (i - j))`` is taken off the scaled score.
     ``sig_bias`` (fp32 [H]): the weights are not a softmax; a visible key weighs ``sigmoid(score + sig_bias)``
-    and nothing is normalised over the keys (no sink then)."""
+    and nothing is normalised over the keys (no sink then).  ``softcap`` c > 0: the scaled score becomes
+    ``c tanh(score / c)`` before masks and softmax; ``keep_first`` n > 0: the window does not hide the keys at
+    positions below n (nothing is renumbered: such keys are addressed by their own positions)."""
     if use_native(qa):
         return native_hybrid().latent_attn_prefill(qa, cache, bt, cu, ctx, window, sink, scale, rk, max_q, mfma, groups,
-                                                   koff, chunk, hscale, ofreq, sig_bias, dist_a, dist_b)
+                                                   koff, chunk, hscale, ofreq, sig_bias, dist_a, dist_b, softcap, keep_first)
     return ref.latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk, groups, koff, chunk, hscale, ofreq,
-                                sig_bias, dist_a, dist_b)
+                                sig_bias, dist_a, dist_b, softcap, keep_first)
 
 
 def latent_attention_decode(qa, cache, bt, ctx, window: int, sink, scale: float, rk: int, mfma: bool = True,
                             groups: int = 1, koff: int = 0, chunk: int = NO_LIMIT, hscale=None, ofreq=None,
-                            max_ctx: int = 0, sig_bias=None, dist_a=None, dist_b=None):
+                            max_ctx: int = 0, sig_bias=None, dist_a=None, dist_b=None, softcap: float = 0.0,
+                            keep_first: int = 0):
     """One query row per sequence, at position ``ctx[n] - 1`` (options as in the prefill form;
     ``max_ctx``: the longest context if the host knows it, it sizes the split of the keys)."""
     if use_native(qa):
         return native_hybrid().latent_attn_decode(qa, cache, bt, ctx, window, sink, scale, rk, mfma, groups, koff, chunk,
-                                                  hscale, ofreq, max_ctx, sig_bias, dist_a, dist_b)
+                                                  hscale, ofreq, max_ctx, sig_bias, dist_a, dist_b, softcap, keep_first)
     cu = torch.arange(qa.shape[0] + 1, dtype=torch.int32)
     return ref.latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk, groups, koff, chunk, hscale, ofreq,
-                                sig_bias, dist_a, dist_b)
+                                sig_bias, dist_a, dist_b, softcap, keep_first)
 
 
 def add_rmsnorm2_f32_(x, a, b, w1, w2, eps: float, one_plus: bool, out_dtype):
@@ -147,14 +150,18 @@ def causal_conv(u, w, state, seq_of, cu, start, sslot, add_input: bool, max_len:
 
 
 def attn_qkv_prep(z, H: int, G: int, dk: int, dv: int, q_norm, k_norm, eps: float, pos, freq, rot_dims: int,
-                  interleaved: bool, amp: float, vfreq, cache, slots):
-    """``z [T, H*dk + G*dk + G*dv] = [q | k | v]``: per-head RMS norm (weights fp32 [dk]) and rotary of
-    q and k, optional turn of v over all of dv by ``position * vfreq``; k and v are written to the
-    token's cache row ``[G, dv + dk] = [v | k]`` at ``slots``; returns q ``[T, H, dk]``."""
+                  interleaved: bool, amp: float, vfreq, cache, slots, v_from_k: bool = False, v_first=None, v_lambda=None):
+    """``z [T, H*dk + G*dk + G*dv] = [q | k | v]``: per-head RMS norm (weights fp32 [dk]; both None: no norm) and
+    rotary of q and k, optional turn of v over all of dv by ``position * vfreq``; k and v are written to the
+    token's cache row ``[G, dv + dk] = [v | k]`` at ``slots``; returns q ``[T, H, dk]``.  ``v_from_k``: ``z = [q | k]``
+    and a token's value is the output of its key projection, taken ahead of norm and rotary (``dv == dk``).  ``v_first`` (``[T, G*dv]``,
+    row-strided views allowed) with ``v_lambda`` (fp32, one number): ``v <- (1 - lambda) v + lambda v_first`` before
+    the write."""
     if use_native(z):
         return native_hybrid().attn_qkv_prep(z, H, G, dk, dv, q_norm, k_norm, eps, pos, freq, rot_dims, interleaved, amp,
-                                             vfreq, cache, slots)
-    return ref.attn_qkv_prep(z, H, G, dk, dv, q_norm, k_norm, eps, pos, freq, rot_dims, interleaved, amp, vfreq, cache, slots)
+                                             vfreq, cache, slots, v_from_k, v_first, v_lambda)
+    return ref.attn_qkv_prep(z, H, G, dk, dv, q_norm, k_norm, eps, pos, freq, rot_dims, interleaved, amp, vfreq, cache, slots,
+                             v_from_k, v_first, v_lambda)
 
 
 def sigmoid_gate_mul(o, g):
@@ -335,13 +342,15 @@ def qk_fullnorm_prep(z, H: int, G: int, dk: int, dv: int, q_norm, k_norm, eps: f
     return ref.qk_fullnorm_prep(z, H, G, dk, dv, q_norm, k_norm, eps, pos, temp_coef, temp_every, cache, slots)
 
 
-def bias_topk_router(logits, bias, top: int):
-    """Softmax scores of ``logits [T, E]`` (fp32); the ``top`` experts with the largest ``score + bias`` are
-    chosen (ties: the lower index); their weights are their own scores (without the bias) over their sum
-    (+ 1e-20).  Returns (expert ids int64 [T, top], weights fp32 [T, top])."""
+def bias_topk_router(logits, bias, top: int, groups: int = 1, keep: int = 1, renorm: bool = True):
+    """Softmax scores of ``logits [T, E]`` (fp32); the ``top`` experts with the largest ``score + bias`` (the
+    choice score; ``bias`` None: the score) are chosen (ties: the lower index).  ``groups`` > 1: the experts
+    form that many equal groups of neighbours, a group's score is its largest choice score, and only experts
+    of the ``keep`` best groups can be chosen.  The weights are the chosen experts' own scores (without the
+    bias), over their sum (+ 1e-20) when ``renorm``.  Returns (expert ids int64 [T, top], weights fp32 [T, top])."""
     if use_native(logits):
-        return native_hybrid().bias_topk_router(logits, bias, top)
-    return ref.bias_topk_router(logits, bias, top)
+        return native_hybrid().bias_topk_router(logits, bias, top, groups, keep, renorm)
+    return ref.bias_topk_router(logits, bias, top, groups, keep, renorm)
 
 
 def act_any(x, kind: str):
@@ -350,3 +359,71 @@ def act_any(x, kind: str):
     if use_native(x):
         return native_hybrid().act_any(x, {"relu2": 0, "gelu": 1}[kind])
     return ref.act_any(x, kind)
+
+
+def hc_embed_norm(ids, table, streams: int, c_in, g, eps: float, out_dtype):
+    """The start of ``streams`` residual streams (hyper-connections): every stream is the embedding row.
+    Returns (``X`` fp32 ``[T, streams, W]``, the first sublayer's input ``norm(sum_s c_in[s] x_s) * g`` ->
+    ``out_dtype``); ``c_in`` fp32 ``[streams]``, ``g`` fp32, one number (an RMS norm with a single weight)."""
+    if use_native(table):
+        return native_hybrid().hc_embed_norm(ids, table, streams, c_in, g, eps, out_dtype == torch.bfloat16)
+    return ref.hc_embed_norm(ids, table, streams, c_in, g, eps, out_dtype)
+
+
+def hc_update_norm_(X, y1, s1: float, y2, s2: float, mix, c_out, mult: float, c_in, g, eps: float, out_dtype):
+    """A sublayer's result into the residual streams ``X`` (fp32 ``[T, S, W]``, in place), all streams at once
+    from the old ones: ``x_t <- sum_s mix[s, t] x_s + mult c_out[t] (s1 y1 + s2 y2)`` (``y2`` may be None; ``y``
+    ``[T, W]`` in the activation dtype or fp32, row-strided views allowed), and the next sublayer's input
+    ``norm(sum_t c_in[t] x_t) * g`` -> ``out_dtype`` in the same pass over the row (None when ``c_in`` is None).
+    One stream with ``mix = c_out = c_in = 1`` is the plain residual sum with a pre-norm."""
+    if use_native(X):
+        h = native_hybrid().hc_update_norm_(X, y1, s1, y2, s2, mix, c_out, mult, c_in, g, eps, out_dtype == torch.bfloat16)
+        return h if c_in is not None else None
+    return ref.hc_update_norm_(X, y1, s1, y2, s2, mix, c_out, mult, c_in, g, eps, out_dtype)
+
+
+def delta_scan(r, k, v, zw, w0, za, ab, decay_coef: float, key_eps: float, S, state_slots, cu, start, cu_host=None, plan=None):
+    """The generalized delta rule over the step's tokens: per head a memory ``S [dk, dv]``; with the decay
+    ``w = exp(-decay_coef sigmoid(zw + w0))`` and the removal rate ``a = sigmoid(za + ab)`` per key channel and the
+    unit key ``u = k / sqrt(sum k^2 + key_eps)``, ``S_t = diag(w_t) S_(t-1) - (a_t u_t) (u_t^T S_(t-1)) + k_t v_t^T``
+    (both terms read the old memory) and ``o_t = S_t^T r_t``.  ``r, k [T, H, dk]``, ``v [T, H, dv]`` (row-strided
+    views allowed), ``zw`` fp32 ``[T, H*dk]``, ``za [T, H*dk]`` (any float dtype), ``w0``, ``ab`` fp32 ``[H*dk]``.
+    Returns fp32 ``[T, H, dv]`` and updates the state pool ``S [slots, H, dk, dv]`` in place at ``state_slots[seq]``
+    (a sequence with ``start == 0`` begins from zeros).  ``plan`` (:func:`gla_chunk_plan` of the row offsets)
+    lets long portions run chunk-parallel."""
+    if use_native(r):
+        nat = native_hybrid()
+        if plan is None and cu_host is not None:
+            plan = gla_chunk_plan(cu_host, r.device)
+        if plan is not None and DELTA_CHUNKED:
+            return _delta_scan_chunked(nat, r, k, v, zw, w0, za, ab, decay_coef, key_eps, S, state_slots, start, plan)
+        return nat.delta_scan(r, k, v, zw, w0, za, ab, decay_coef, key_eps, S, state_slots, cu, start, None, True, True)
+    return ref.delta_scan(r, k, v, zw, w0, za, ab, decay_coef, key_eps, S, state_slots, cu, start)
+
+
+DELTA_CHUNKED = False
+
+
+def tanh_act(x):
+    """Elementwise ``tanh`` (computed in fp32) -> x's dtype."""
+    if use_native(x):
+        return native_hybrid().tanh_act(x.contiguous())
+    return ref.tanh_act(x)
+
+
+def softcap_(x, cap: float):
+    """``x <- cap tanh(x / cap)`` in place on an fp32 tensor."""
+    if use_native(x):
+        native_hybrid().softcap_(x, cap)
+        return x
+    return ref.softcap_(x, cap)
+
+
+
+def gated_add_f32_(out, y, g):
+    """``out += y * sigmoid(g)`` in place on the fp32 ``out [T, W]``; ``y [T, W]`` in any float dtype, ``g [T, 1]``
+    one gate logit per row (row-strided views allowed)."""
+    if use_native(out):
+        native_hybrid().gated_add_f32_(out, y, g)
+        return out
+    return ref.gated_add_f32_(out, y, g)

@@ -61,7 +61,7 @@ def latent_q_assemble(q_lat, q, pos, inv_freq, rot_dims, dn, interleaved=False, 
 
 
 def latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk, groups=1, koff=0, chunk=1 << 30, hscale=None,
-                     ofreq=None, sig_bias=None, dist_a=None, dist_b=None):
+                     ofreq=None, sig_bias=None, dist_a=None, dist_b=None, softcap=0.0, keep_first=0):
     """Attention over a paged row cache.  Sequence n owns query rows [cu[n], cu[n+1]); its last query
     sits at position ctx[n] - 1.  A token's cache row holds ``groups`` sub-rows; query head h reads
     sub-row h / (H / groups), whose entries [koff, koff + R) are the key and whose first ``rk`` entries
@@ -69,7 +69,9 @@ def latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk, groups=1, 
     its window (i - j < window) and its chunk (i // chunk == j // chunk); ``sink`` [H] joins the softmax
     denominator; ``hscale`` [H] multiplies the scores; ``ofreq`` [rk / 2] turns the output's neighbour
     pairs back by -position * ofreq.  ``dist_a``, ``dist_b`` [H]: ``dist_a ln(1 + dist_b (i - j))`` is taken
-    off the scaled score; ``sig_bias`` [H]: no softmax, a visible key weighs sigmoid(score + sig_bias)."""
+    off the scaled score; ``sig_bias`` [H]: no softmax, a visible key weighs sigmoid(score + sig_bias).
+    ``softcap`` c > 0: the scaled score becomes c tanh(score / c); ``keep_first`` n: the window does not hide
+    the keys at positions below n."""
     T, H, R = qa.shape
     bs = cache.shape[1]
     G = groups
@@ -84,13 +86,17 @@ def latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk, groups=1, 
             continue
         p0 = ctx_l[n] - (b - a)  # position of the first query row
         lo = max(0, p0 - window + 1, (p0 // chunk) * chunk)
+        if keep_first > 0:
+            lo = max(0, (p0 // chunk) * chunk)
         kpos = torch.arange(lo, ctx_l[n])
         rows = flat[bt[n, (kpos // bs).long()].long() * bs + kpos % bs].float()  # [K, G, rs]
         rows = rows.repeat_interleave(H // G, 1)  # [K, H, rs]
         s = torch.einsum("thr,khr->htk", qa[a:b].float(), rows[:, :, koff:koff + R]) * scale * hs
+        if softcap > 0.0:
+            s = softcap * torch.tanh(s / softcap)
         qpos = torch.arange(p0, ctx_l[n])
         d = qpos[:, None] - kpos[None, :]
-        vis = (d >= 0) & (d < window) & (qpos[:, None] // chunk == kpos[None, :] // chunk)
+        vis = (d >= 0) & ((d < window) | (kpos[None, :] < keep_first)) & (qpos[:, None] // chunk == kpos[None, :] // chunk)
         if dist_a is not None:
             s = s - dist_a.float().view(H, 1, 1) * torch.log1p(dist_b.float().view(H, 1, 1) * d.clamp(min=0).float())
         if sig_bias is not None:
@@ -155,16 +161,24 @@ def causal_conv(u, w, state, seq_of, cu, start, sslot, add_input):
     return y.to(u.dtype)
 
 
-def attn_qkv_prep(z, H, G, dk, dv, q_norm, k_norm, eps, pos, freq, rot_dims, interleaved, amp, vfreq, cache, slots):
-    """z [T, H*dk + G*dk + G*dv] = [q | k | v]: per-head RMS norm and rotary of q and k, optional turn of
-    v over all of dv; k and v go to the token's cache row [G, dv + dk] = [v | k]; returns q [T, H, dk]."""
+def attn_qkv_prep(z, H, G, dk, dv, q_norm, k_norm, eps, pos, freq, rot_dims, interleaved, amp, vfreq, cache, slots,
+                  v_from_k=False, v_first=None, v_lambda=None):
+    """z [T, H*dk + G*dk + G*dv] = [q | k | v]: per-head RMS norm (skipped when the weights are None) and rotary
+    of q and k, optional turn of v over all of dv; k and v go to the token's cache row [G, dv + dk] = [v | k];
+    returns q [T, H, dk].  ``v_from_k``: z = [q | k] and the value is the key projection's output (ahead of norm and
+    rotary).  ``v_first`` [T, G*dv] with ``v_lambda`` (one number): v <- (1 - lambda) v + lambda v_first."""
     T = z.shape[0]
     zf = z.float()
     q, k = zf[:, :H * dk].view(T, H, dk), zf[:, H * dk:(H + G) * dk].view(T, G, dk)
-    v = zf[:, (H + G) * dk:].view(T, G, dv)
+    v = k if v_from_k else zf[:, (H + G) * dk:(H + G) * dk + G * dv].view(T, G, dv)
+    if v_first is not None:
+        lam = v_lambda.float().reshape(())
+        v = (1.0 - lam) * v + lam * v_first.float().view(T, G, dv)
     unit = lambda x: x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
-    q = _rotate(unit(q) * q_norm.float(), pos, freq, rot_dims, interleaved, amp)
-    k = _rotate(unit(k) * k_norm.float(), pos, freq, rot_dims, interleaved, amp)
+    if q_norm is not None:
+        q, k = unit(q) * q_norm.float(), unit(k) * k_norm.float()
+    q = _rotate(q, pos, freq, rot_dims, interleaved, amp)
+    k = _rotate(k, pos, freq, rot_dims, interleaved, amp)
     if vfreq is not None:
         v = _rotate(v, pos, vfreq, dv, interleaved)
     row = torch.cat([v, k], -1).reshape(T, G * (dv + dk)).to(cache.dtype)
@@ -293,11 +307,18 @@ def qk_fullnorm_prep(z, H, G, dk, dv, q_norm, k_norm, eps, pos, temp_coef, temp_
     return q.view(T, H, dk).to(z.dtype)
 
 
-def bias_topk_router(logits, bias, top):
+def bias_topk_router(logits, bias, top, groups=1, keep=1, renorm=True):
     s = torch.softmax(logits.float(), -1)
-    idx = (s + bias.float()).topk(top, -1).indices
+    c = s + bias.float() if bias is not None else s
+    if groups > 1:
+        T, E = c.shape
+        per = E // groups
+        best = c.view(T, groups, per).max(-1).values.topk(keep, -1).indices
+        ok = torch.zeros(T, groups, dtype=torch.bool).scatter_(1, best, True)
+        c = c.masked_fill(~ok[:, :, None].expand(T, groups, per).reshape(T, E), float("-inf"))
+    idx = c.topk(top, -1).indices
     w = s.gather(1, idx)
-    return idx, w / (w.sum(-1, keepdim=True) + 1e-20)
+    return idx, (w / (w.sum(-1, keepdim=True) + 1e-20) if renorm else w)
 
 
 def act_any(x, kind):
@@ -309,3 +330,68 @@ def act_any(x, kind):
     else:
         raise ValueError(f"unknown activation {kind!r}")
     return y.to(x.dtype)
+
+
+def hc_embed_norm(ids, table, streams, c_in, g, eps, out_dtype):
+    """Every one of ``streams`` residual streams starts as the embedding; returns (X fp32 [T, S, W], the first
+    sublayer's input ``norm(sum_s c_in[s] x_s) * g``)."""
+    x = table[ids].float()
+    X = x[:, None, :].repeat(1, streams, 1).contiguous()
+    u = x * c_in.float().sum()
+    return X, (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * g.float().reshape(())).to(out_dtype)
+
+
+def hc_update_norm_(X, y1, s1, y2, s2, mix, c_out, mult, c_in, g, eps, out_dtype):
+    """A sublayer's result into ``streams`` residual streams X fp32 [T, S, W], all at once from the old ones:
+    ``x_t <- sum_s mix[s, t] x_s + mult c_out[t] (s1 y1 + s2 y2)``; then, when ``c_in`` is given, the next
+    sublayer's input ``norm(sum_t c_in[t] x_t) * g`` (else None)."""
+    y = y1.float() * s1
+    if y2 is not None:
+        y = y + y2.float() * s2
+    new = torch.einsum("st,nsw->ntw", mix.float(), X) + mult * c_out.float()[None, :, None] * y[:, None, :]
+    X.copy_(new)
+    if c_in is None:
+        return None
+    u = torch.einsum("t,ntw->nw", c_in.float(), X)
+    return (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * g.float().reshape(())).to(out_dtype)
+
+
+def delta_scan(r, k, v, zw, w0, za, ab, decay_coef, key_eps, S, state_slots, cu, start):
+    """Token-by-token generalized delta rule.  Per head a memory S [dk, dv]: with the decay ``w = exp(-decay_coef
+    sigmoid(zw + w0))``, the removal rate ``a = sigmoid(za + ab)`` and the unit key ``u = k / sqrt(sum k^2 + key_eps)``,
+    ``S_t = diag(w) S_(t-1) - (a u) (u^T S_(t-1)) + k v^T`` and ``o_t = S_t^T r``.  The state pool S [slots, H, dk, dv]
+    (fp32) is read at ``state_slots[seq]`` (zeros when the sequence starts at position 0) and written back after
+    the sequence's last token of this step."""
+    T, H, dk = r.shape
+    dv = v.shape[-1]
+    out = torch.zeros(T, H, dv, dtype=torch.float32)
+    w = torch.exp(-decay_coef * torch.sigmoid(zw.float() + w0.float())).view(T, H, dk)
+    a = torch.sigmoid(za.float() + ab.float()).view(T, H, dk)
+    kf = k.float()
+    u = kf * torch.rsqrt(kf.pow(2).sum(-1, keepdim=True) + key_eps)
+    cu_l = [int(x) for x in cu]
+    for s in range(len(cu_l) - 1):
+        lo, hi = cu_l[s], cu_l[s + 1]
+        if lo == hi:
+            continue
+        slot = int(state_slots[s])
+        Ss = torch.zeros_like(S[slot]) if int(start[s]) == 0 else S[slot].clone()
+        for t in range(lo, hi):
+            uS = torch.einsum("hk,hkv->hv", u[t], Ss)
+            Ss = w[t][:, :, None] * Ss - (a[t] * u[t])[:, :, None] * uS[:, None, :] + kf[t][:, :, None] * v[t].float()[:, None, :]
+            out[t] = torch.einsum("hkv,hk->hv", Ss, r[t].float())
+        S[slot] = Ss
+    return out
+
+
+def tanh_act(x):
+    return torch.tanh(x.float()).to(x.dtype)
+
+
+def softcap_(x, cap):
+    return x.copy_(cap * torch.tanh(x / cap))
+
+
+def gated_add_f32_(out, y, g):
+    out += y.float() * torch.sigmoid(g.float())
+    return out
