@@ -115,6 +115,8 @@ struct RowAttnOpts {
   const float* dist_a = nullptr;      // [H], with dist_b [H]: dist_a ln(1 + dist_b (i - j)) is taken off the scaled score
   const float* dist_b = nullptr;
   const float* sig_bias = nullptr;    // [H]: no softmax; a visible key weighs sigmoid(score + sig_bias), nothing is normalised
+  double softcap = 0.0;               // c > 0: the scaled score becomes c tanh(score / c)
+  int64_t keep_first = 0;             // the window does not hide the keys at positions below this
 };
 
 }  // namespace llmctl_hybrid

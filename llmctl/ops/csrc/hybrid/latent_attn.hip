@@ -96,8 +96,8 @@ struct GenArgs {
   const float* dist_a;  // nullptr: no distance penalty
   const float* dist_b;
   const float* sig_bias;  // SIG forms: the head's bias inside the sigmoid
-  int bt_stride, H, R, rk, bs, window, chunk, G, rs, koff;
-  float scale;
+  int bt_stride, H, R, rk, bs, window, chunk, G, rs, koff, keep;  // keep: the window spares the keys at positions below it
+  float scale, cap, inv_cap;                                       // cap > 0: the scaled score becomes cap tanh(score / cap)
 };
 
 __device__ __forceinline__ int first_visible(int p, int window, int chunk) { return max(max(p - window + 1, (p / chunk) * chunk), 0); }
@@ -123,6 +123,11 @@ __global__ __launch_bounds__(64) void latent_attn_prefill_kernel(const T* __rest
   const int last = p0 + min(q0 + 63, qlen - 1);
   const int j0 = first_visible(p0 + q0, g.window, g.chunk);
   const int lo = first_visible(qp, g.window, g.chunk);
+  // keys that the window spares: positions [c0, min(keep, j0)) of the chunk of the tile's first query (a tile that
+  // spans two chunks starts the second one inside [j0, last], where the chunk test below applies)
+  const int c0 = ((p0 + q0) / g.chunk) * g.chunk;
+  const int kept = max(min(g.keep, j0) - c0, 0);
+  const int cq = (qp / g.chunk) * g.chunk;  // first position of this query's chunk
   const float scale = g.scale * (g.hscale != nullptr ? g.hscale[h] : 1.0f);
   const bool pen = g.dist_a != nullptr;
   const float da = pen ? g.dist_a[h] : 0.f, db = pen ? g.dist_b[h] : 0.f;
@@ -137,13 +142,15 @@ __global__ __launch_bounds__(64) void latent_attn_prefill_kernel(const T* __rest
   for (int i = 0; i < VT; ++i) acc[i] = 0.f;
   const int* btn = g.bt + (int64_t)n * g.bt_stride;
   const int grp = h / (H / g.G);
-  for (int j = j0; j <= last; ++j) {
+  for (int jj = -kept; jj <= last - j0; ++jj) {
+    const int j = jj < 0 ? c0 + kept + jj : j0 + jj;
     const T* row = cache + (((int64_t)btn[j / bs] * bs + j % bs) * g.G + grp) * g.rs;
     const T* key = row + g.koff;
     float s = 0.f;
     for (int d = 0; d < R; ++d) s += qT[d * 64 + lane] * ldf(key + d);
     s *= scale;
-    if (live && j <= qp && j >= lo) {
+    if (g.cap > 0.f) s = g.cap * tanhf(s * g.inv_cap);
+    if (live && j <= qp && (j >= lo || (j < g.keep && j >= cq))) {
       if (pen) s -= da * log1pf(db * (float)(qp - j));
       if constexpr (SIG) {
         const float p = 1.0f / (1.0f + expf(-(s + sb)));
@@ -194,7 +201,9 @@ __global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __rest
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int len = g.ctx[n];
   const int lo = first_visible(len - 1, g.window, g.chunk);
-  const int nk = len - lo;
+  const int c0 = ((len - 1) / g.chunk) * g.chunk;
+  const int kept = max(min(g.keep, lo) - c0, 0);  // keys before the window that it spares: [c0, c0 + kept)
+  const int nk = kept + len - lo;
   const T* qr = qa + ((int64_t)n * H + h) * R;
   for (int d = threadIdx.x; d < R; d += 256) qs[d] = ldf(qr + d);
   __syncthreads();
@@ -209,8 +218,9 @@ __global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __rest
 #pragma unroll
   for (int i = 0; i < NA; ++i) acc[i] = 0.f;
   for (int c = wave * 64; c < nk; c += 256) {
-    const int j = lo + c + lane;
-    const bool ok = c + lane < nk;
+    const int ci = c + lane;
+    const int j = ci < kept ? c0 + ci : lo + ci - kept;
+    const bool ok = ci < nk;
     int64_t slot = 0;
     float s = -INFINITY;
     if (ok) {
@@ -219,6 +229,7 @@ __global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __rest
       float d0 = 0.f;
       for (int d = 0; d < R; ++d) d0 += qs[d] * ldf(key + d);
       s = d0 * scale;
+      if (g.cap > 0.f) s = g.cap * tanhf(s * g.inv_cap);
       if (pen) s -= da * log1pf(db * (float)(len - 1 - j));
     }
     float p, corr;
@@ -294,6 +305,10 @@ __global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __rest
 
 // latent_attn_mfma.hip: the matrix-core form for bf16 shapes that fit it
 bool latent_attn_mfma_ok(const at::Tensor& qa, int64_t rk, int64_t rs, int64_t koff, bool turn_back);
+// capped scores are built into the plain softmax form only, for keys up to 256 wide
+static bool mfma_cap_ok(const RowAttnOpts& x, int64_t R) {
+  return x.softcap == 0.0 || (x.ofreq == nullptr && x.sig_bias == nullptr && x.hscale == nullptr && R <= 256);
+}
 void latent_attn_mfma(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor* cu, const at::Tensor& ctx,
                       int64_t window, const float* sink, double scale, int64_t rk, int64_t max_q, at::Tensor& out, const RowAttnOpts& x);
 
@@ -356,7 +371,8 @@ at::Tensor latent_q_assemble(const at::Tensor& q_lat, const at::Tensor& q, const
 static RowAttnOpts row_opts(const at::Tensor& qa, const at::Tensor& cache, int64_t rk, const c10::optional<at::Tensor>& sink, int64_t groups,
                             int64_t koff, int64_t chunk, const c10::optional<at::Tensor>& hscale, const c10::optional<at::Tensor>& ofreq,
                             int64_t max_ctx, const float** sink_p, const c10::optional<at::Tensor>& sig_bias = c10::nullopt,
-                            const c10::optional<at::Tensor>& dist_a = c10::nullopt, const c10::optional<at::Tensor>& dist_b = c10::nullopt) {
+                            const c10::optional<at::Tensor>& dist_a = c10::nullopt, const c10::optional<at::Tensor>& dist_b = c10::nullopt,
+                            double softcap = 0.0, int64_t keep_first = 0) {
   const int64_t H = qa.size(1), R = qa.size(2);
   HYB_CHECK(groups >= 1 && H % groups == 0 && cache.size(2) % groups == 0, "kv groups must divide the heads and the cache row");
   const int64_t rs = cache.size(2) / groups;
@@ -379,6 +395,9 @@ static RowAttnOpts row_opts(const at::Tensor& qa, const at::Tensor& cache, int64
   x.dist_a = dist_a.has_value() ? dist_a->data_ptr<float>() : nullptr;
   x.dist_b = dist_b.has_value() ? dist_b->data_ptr<float>() : nullptr;
   x.sig_bias = sig_bias.has_value() ? sig_bias->data_ptr<float>() : nullptr;
+  HYB_CHECK(softcap >= 0.0 && keep_first >= 0, "softcap >= 0, keep_first >= 0");
+  x.softcap = softcap;
+  x.keep_first = std::min<int64_t>(keep_first, (int64_t)1 << 30);
   return x;
 }
 
@@ -403,7 +422,10 @@ static GenArgs gen_args(const at::Tensor& qa, const at::Tensor& cache, const at:
   g.G = (int)x.groups;
   g.rs = (int)(cache.size(2) / x.groups);
   g.koff = (int)x.koff;
+  g.keep = (int)x.keep_first;
   g.scale = (float)scale;
+  g.cap = (float)x.softcap;
+  g.inv_cap = x.softcap > 0.0 ? (float)(1.0 / x.softcap) : 0.f;
   return g;
 }
 
@@ -412,7 +434,7 @@ at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, co
                                int64_t max_q, bool mfma, int64_t groups, int64_t koff, int64_t chunk,
                                const c10::optional<at::Tensor>& hscale, const c10::optional<at::Tensor>& ofreq,
                                const c10::optional<at::Tensor>& sig_bias, const c10::optional<at::Tensor>& dist_a,
-                               const c10::optional<at::Tensor>& dist_b) {
+                               const c10::optional<at::Tensor>& dist_b, double softcap, int64_t keep_first) {
   HYB_CHECK(qa.is_cuda() && qa.is_contiguous() && qa.dim() == 3, "qa: contiguous [T, H, R]");
   const int64_t T = qa.size(0), H = qa.size(1), R = qa.size(2);
   check_cache(cache, qa, cache.size(2));
@@ -424,12 +446,12 @@ at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, co
   HYB_CHECK(window >= 1 && max_q >= 1, "window >= 1, max_q >= 1");
   window = std::min<int64_t>(window, (int64_t)1 << 30);
   const float* sink_p;
-  const RowAttnOpts x = row_opts(qa, cache, rk, sink, groups, koff, chunk, hscale, ofreq, 0, &sink_p, sig_bias, dist_a, dist_b);
+  const RowAttnOpts x = row_opts(qa, cache, rk, sink, groups, koff, chunk, hscale, ofreq, 0, &sink_p, sig_bias, dist_a, dist_b, softcap, keep_first);
   HYB_CHECK((size_t)R * 64 * sizeof(float) <= 160 * 1024, "key too wide for the query tile in LDS");
   c10::DeviceGuard guard(qa.device());
   at::Tensor out = at::empty({T, H, rk}, qa.options());
   if (T == 0 || ns == 0) return out;
-  if (mfma && (x.dist_a == nullptr || x.sig_bias != nullptr) && latent_attn_mfma_ok(qa, rk, cache.size(2) / groups, koff, x.ofreq != nullptr || x.sig_bias != nullptr)) {
+  if (mfma && mfma_cap_ok(x, R) && (x.dist_a == nullptr || x.sig_bias != nullptr) && latent_attn_mfma_ok(qa, rk, cache.size(2) / groups, koff, x.ofreq != nullptr || x.sig_bias != nullptr)) {
     latent_attn_mfma(qa, cache, bt, &cu, ctx, window, sink_p, scale, rk, max_q, out, x);
     return out;
   }
@@ -462,7 +484,7 @@ at::Tensor latent_attn_decode(const at::Tensor& qa, const at::Tensor& cache, con
                               int64_t window, const c10::optional<at::Tensor>& sink, double scale, int64_t rk, bool mfma, int64_t groups,
                               int64_t koff, int64_t chunk, const c10::optional<at::Tensor>& hscale, const c10::optional<at::Tensor>& ofreq,
                               int64_t max_ctx, const c10::optional<at::Tensor>& sig_bias, const c10::optional<at::Tensor>& dist_a,
-                              const c10::optional<at::Tensor>& dist_b) {
+                              const c10::optional<at::Tensor>& dist_b, double softcap, int64_t keep_first) {
   HYB_CHECK(qa.is_cuda() && qa.is_contiguous() && qa.dim() == 3, "qa: contiguous [n, H, R]");
   const int64_t ns = qa.size(0), H = qa.size(1), R = qa.size(2);
   check_cache(cache, qa, cache.size(2));
@@ -472,11 +494,11 @@ at::Tensor latent_attn_decode(const at::Tensor& qa, const at::Tensor& cache, con
   HYB_CHECK(window >= 1, "window >= 1");
   window = std::min<int64_t>(window, (int64_t)1 << 30);
   const float* sink_p;
-  const RowAttnOpts x = row_opts(qa, cache, rk, sink, groups, koff, chunk, hscale, ofreq, max_ctx, &sink_p, sig_bias, dist_a, dist_b);
+  const RowAttnOpts x = row_opts(qa, cache, rk, sink, groups, koff, chunk, hscale, ofreq, max_ctx, &sink_p, sig_bias, dist_a, dist_b, softcap, keep_first);
   c10::DeviceGuard guard(qa.device());
   at::Tensor out = at::empty({ns, H, rk}, qa.options());
   if (ns == 0) return out;
-  if (mfma && (x.dist_a == nullptr || x.sig_bias != nullptr) && latent_attn_mfma_ok(qa, rk, cache.size(2) / groups, koff, x.ofreq != nullptr || x.sig_bias != nullptr)) {
+  if (mfma && mfma_cap_ok(x, R) && (x.dist_a == nullptr || x.sig_bias != nullptr) && latent_attn_mfma_ok(qa, rk, cache.size(2) / groups, koff, x.ofreq != nullptr || x.sig_bias != nullptr)) {
     latent_attn_mfma(qa, cache, bt, nullptr, ctx, window, sink_p, scale, rk, 1, out, x);
     return out;
   }

@@ -42,7 +42,9 @@ struct LArgs {
   const float* sig_bias;
   int H, R, rk, bs, maxb, window, HB, nvt;
   int G, rs, koff, chunk, hpg;  // kv groups, row width, key's first column, chunk mask size, head tiles per group
+  int keep;                     // the window spares the keys at positions below this
   float scale_log2;
+  float cap_log2, cap_inv2;     // CAP forms: x (log2 domain) = cap_log2 * tanh(s * scale); cap_inv2 = 2 log2(e) scale / cap
   // decode rows with the key range split over blockIdx.x (few sequences would otherwise leave the chip
   // idle): each split writes its unnormalised fp32 output and (running maximum, denominator) here
   int nsplit;
@@ -53,8 +55,9 @@ struct LArgs {
 // ROT: the output's neighbour pairs are turned back by the query's position (a.ofreq); a template flag
 // so that the forms without it keep their register budget.  SIG: the weights are sigmoids of the scores
 // (after the distance penalty), not a softmax: no running maximum, no rescale, no denominator; the splits
-// of decode rows are merged as a plain sum (m = 0 everywhere, l = 1 in the first split only).
-template <int NCB, int NDB, bool ROT, bool SIG = false>
+// of decode rows are merged as a plain sum (m = 0 everywhere, l = 1 in the first split only).  CAP: the scaled score
+// s becomes cap tanh(s / cap) before masks and softmax (tanh y = 1 - 2 / (1 + e^(2y))).
+template <int NCB, int NDB, bool ROT, bool SIG = false, bool CAP = false>
 __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   constexpr int NKS = NCB * 8;
   constexpr int NTB = (NDB + 3) / 4;
@@ -124,7 +127,14 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   const int first_pos = pos0 + tok0, last_pos = pos0 + min(tok0 + TB, qlen) - 1;
   // the first key a query at position p may see: inside its window and inside its chunk
   auto first_key = [&](int p) { return max(max(p - a.window + 1, (p / a.chunk) * a.chunk), 0); };
-  int t_lo = first_key(first_pos) / LKB, t_hi = last_pos / LKB + 1;
+  const int t_first = first_key(first_pos) / LKB, t_end = last_pos / LKB + 1;
+  // tiles before the window whose first keys it spares (those of the chunk of the block's first row; a block that
+  // spans two chunks meets the second one inside the window's tiles): the key loop runs over them first.  Loop
+  // index i in [t_lo, t_hi) stands for tile i < n_kept ? kept0 + i : t_first + i - n_kept.
+  const int kept0 = ((first_pos / a.chunk) * a.chunk) / LKB;
+  const int n_kept = a.keep > 0 ? max(min((a.keep + LKB - 1) / LKB, t_first) - kept0, 0) : 0;
+  auto tile_of = [&](int i) { return i < n_kept ? kept0 + i : t_first + i - n_kept; };
+  int t_lo = 0, t_hi = n_kept + t_end - t_first;
   if (a.nsplit > 1) {
     const int per = (t_hi - t_lo + a.nsplit - 1) / a.nsplit;
     t_lo += split * per;
@@ -135,6 +145,7 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   const int w_last = pos0 + min(tok0 + (wave * 32 + 31) / HB, qlen - 1);
   const bool wave_live = tok0 + (wave * 32) / HB < qlen && hsub + (HB >= 32 ? (wave * 32) % HB : 0) < P;
   const int w_lo = first_key(w_first), my_lo = first_key(my_pos);
+  const int my_c0 = (my_pos / a.chunk) * a.chunk;  // first position of this row's chunk
   const int w_lo_last = first_key(w_last);  // first_key never decreases with the position
   // lane-only parts of the LDS read addresses, so that the key loop adds constants to them
   int tr_lo[4], tr_hi[4];
@@ -181,11 +192,11 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
     return btn[key / a.bs] * a.bs + key % a.bs;
   };
   int pend = 0;
-  if (t_lo < t_hi) load_slots(t_lo, 0);
+  if (t_lo < t_hi) load_slots(tile_of(t_lo), 0);
   if constexpr (DB) {
     if (t_lo < t_hi) {
       __syncthreads();
-      if (t_lo + 1 < t_hi && tid < LKB) pend = slot_of(t_lo + 1);
+      if (t_lo + 1 < t_hi && tid < LKB) pend = slot_of(tile_of(t_lo + 1));
       fill(0, 0);
     }
   }
@@ -199,17 +210,17 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
       if (t + 1 < t_hi && tid < LKB) slot_lds[(sbuf ^ 1) * LKB + tid] = pend;
       vm_wait<0>();
       __syncthreads();
-      if (t + 2 < t_hi && tid < LKB) pend = slot_of(t + 2);
+      if (t + 2 < t_hi && tid < LKB) pend = slot_of(tile_of(t + 2));
       if (t + 1 < t_hi) fill(sbuf ^ 1, sbuf ^ 1);
     } else {
       __syncthreads();
       fill(sbuf, 0);
-      if (t + 1 < t_hi) load_slots(t + 1, sbuf ^ 1);
+      if (t + 1 < t_hi) load_slots(tile_of(t + 1), sbuf ^ 1);
       vm_wait<0>();
       __syncthreads();
     }
-    const int kv0 = t * LKB;
-    if (!wave_live || kv0 > w_last || kv0 + LKB - 1 < w_lo) continue;
+    const int kv0 = tile_of(t) * LKB;
+    if (!wave_live || kv0 > w_last || (kv0 + LKB - 1 < w_lo && kv0 >= a.keep)) continue;
 
     f32x16 s[2];
 #pragma unroll
@@ -234,7 +245,7 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
           const float dist = (float)max(my_pos - key, 0);
           const float x = s[kb][i] * my_scale - pen_a * __log2f(1.0f + pen_b * dist) + sig_b2;
           const float w = __builtin_amdgcn_rcpf(1.0f + fast_exp2(-x));
-          p[i] = (!valid || key > my_pos || key < my_lo || key >= ctx) ? 0.f : w;
+          p[i] = (!valid || key > my_pos || (key < my_lo && (key >= a.keep || key < my_c0)) || key >= ctx) ? 0.f : w;
         }
         pb[kb][0] = to_bf16x8(p);
         pb[kb][1] = to_bf16x8(p + 8);
@@ -248,7 +259,8 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
-            s[kb][i] *= my_scale;
+            if constexpr (CAP) s[kb][i] = a.cap_log2 * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + fast_exp2(s[kb][i] * a.cap_inv2)));
+            else s[kb][i] *= my_scale;
             mx = fmaxf(mx, s[kb][i]);
           }
         if (!valid) mx = -INFINITY;  // such a row must not trigger the wave's rescale
@@ -257,9 +269,11 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
-            float x = s[kb][i] * my_scale;
+            float x;
+            if constexpr (CAP) x = a.cap_log2 * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + fast_exp2(s[kb][i] * a.cap_inv2)));
+            else x = s[kb][i] * my_scale;
             const int key = kv0 + kb * 32 + acc_row(i, hh);
-            if (!valid || key > my_pos || key < my_lo || key >= ctx) x = -INFINITY;
+            if (!valid || key > my_pos || (key < my_lo && (key >= a.keep || key < my_c0)) || key >= ctx) x = -INFINITY;
             s[kb][i] = x;
             mx = fmaxf(mx, x);
           }
@@ -374,7 +388,7 @@ __global__ void latent_split_merge_kernel(const float* __restrict__ ws_o, const 
   }
 }
 
-template <int NCB, bool ROT, bool SIG = false>
+template <int NCB, bool ROT, bool SIG = false, bool CAP = false>
 void launch_ncb(const LArgs& a, int ndb, dim3 grid, hipStream_t st) {
   auto go = [&](auto kern, int NDBv) {
     const size_t one = (size_t)(NCB + (NDBv + 3) / 4) * LIMG;
@@ -382,9 +396,9 @@ void launch_ncb(const LArgs& a, int ndb, dim3 grid, hipStream_t st) {
     HYB_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess, "LDS size");
     kern<<<grid, 256, lds, st>>>(a);
   };
-  if (ndb == 2) go(latent_attn_mfma_kernel<NCB, 2, ROT, SIG>, 2);
-  else if (ndb == 4) go(latent_attn_mfma_kernel<NCB, 4, ROT, SIG>, 4);
-  else go(latent_attn_mfma_kernel<NCB, 8, ROT, SIG>, 8);
+  if (ndb == 2) go(latent_attn_mfma_kernel<NCB, 2, ROT, SIG, CAP>, 2);
+  else if (ndb == 4) go(latent_attn_mfma_kernel<NCB, 4, ROT, SIG, CAP>, 4);
+  else go(latent_attn_mfma_kernel<NCB, 8, ROT, SIG, CAP>, 8);
 }
 }  // namespace
 
@@ -416,7 +430,7 @@ void latent_attn_mfma(const at::Tensor& qa, const at::Tensor& cache, const at::T
   at::Tensor ws_o, ws_ml;
   if (cu == nullptr && rk % 4 == 0) {
     const int64_t span = std::min<int64_t>(std::min<int64_t>(window, x.chunk), x.max_ctx > 0 ? x.max_ctx : (int64_t)1 << 30);
-    const int tiles = (int)std::min<int64_t>((span + LKB - 1) / LKB + 1, 1 << 20);
+    const int tiles = (int)std::min<int64_t>((span + LKB - 1) / LKB + 1 + (x.keep_first + LKB - 1) / LKB, 1 << 20);
     const long blocks = (long)ns * hgroups * nvt;
     while (nsplit < tiles && nsplit < 32 && blocks * nsplit < 512) nsplit *= 2;
     if (nsplit > 1) {
@@ -427,12 +441,17 @@ void latent_attn_mfma(const at::Tensor& qa, const at::Tensor& cache, const at::T
   LArgs a{reinterpret_cast<const unsigned short*>(qa.data_ptr()), reinterpret_cast<const unsigned short*>(cache.data_ptr()),
           reinterpret_cast<unsigned short*>(out.data_ptr()), bt.data_ptr<int>(), cu ? cu->data_ptr<int>() : nullptr, ctx.data_ptr<int>(),
           sink, x.hscale, x.ofreq, x.dist_a, x.dist_b, x.sig_bias, (int)H, (int)R, (int)rk, (int)cache.size(1), (int)bt.size(1), (int)window, HB, nvt,
-          (int)G, (int)rs, (int)x.koff, (int)x.chunk, hpg,
-          (float)(scale * 1.4426950408889634), nsplit, nsplit > 1 ? ws_o.data_ptr<float>() : nullptr,
+          (int)G, (int)rs, (int)x.koff, (int)x.chunk, hpg, (int)x.keep_first,
+          (float)(scale * 1.4426950408889634), (float)(x.softcap * 1.4426950408889634),
+          x.softcap > 0.0 ? (float)(2.0 * 1.4426950408889634 * scale / x.softcap) : 0.f, nsplit, nsplit > 1 ? ws_o.data_ptr<float>() : nullptr,
           nsplit > 1 ? ws_ml.data_ptr<float>() : nullptr};
   dim3 grid(nsplit > 1 ? (unsigned)nsplit : (unsigned)((max_q + TB - 1) / TB), (unsigned)ns, (unsigned)(hgroups * nvt));
   hipStream_t st = cur_stream();
-  if (x.sig_bias != nullptr) {  // built for keys up to 256 wide (latent_attn_mfma_ok)
+  if (x.softcap > 0.0) {  // built for keys up to 256 wide, plain softmax form (the caller checks)
+    HYB_CHECK(x.hscale == nullptr && ncb <= 2, "capped scores: no per-head factor, keys up to 256 wide");
+    if (ncb == 1) launch_ncb<1, false, false, true>(a, ndb, grid, st);
+    else launch_ncb<2, false, false, true>(a, ndb, grid, st);
+  } else if (x.sig_bias != nullptr) {  // built for keys up to 256 wide (latent_attn_mfma_ok)
     if (ncb == 1) launch_ncb<1, false, true>(a, ndb, grid, st);
     else launch_ncb<2, false, true>(a, ndb, grid, st);
   } else if (x.ofreq != nullptr) {

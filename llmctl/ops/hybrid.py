@@ -395,13 +395,32 @@ def delta_scan(r, k, v, zw, w0, za, ab, decay_coef: float, key_eps: float, S, st
         nat = native_hybrid()
         if plan is None and cu_host is not None:
             plan = gla_chunk_plan(cu_host, r.device)
-        if plan is not None and DELTA_CHUNKED:
+        if plan is not None and DELTA_CHUNKED and k.shape[2] * v.shape[2] <= DELTA_COMBINE_MAX:
             return _delta_scan_chunked(nat, r, k, v, zw, w0, za, ab, decay_coef, key_eps, S, state_slots, start, plan)
         return nat.delta_scan(r, k, v, zw, w0, za, ab, decay_coef, key_eps, S, state_slots, cu, start, None, True, True)
     return ref.delta_scan(r, k, v, zw, w0, za, ab, decay_coef, key_eps, S, state_slots, cu, start)
 
 
-DELTA_CHUNKED = False
+DELTA_CHUNKED = True  # long portions run chunk-parallel
+DELTA_COMBINE_MAX = 8192  # memory entries per head that the combine pass holds twice in LDS
+
+
+def _delta_scan_chunked(nat, r, k, v, zw, w0, za, ab, decay_coef, key_eps, S, state_slots, start, plan):
+    """The same recurrence with the chunks of a portion side by side.  The memory is linear in its past: a token
+    maps it by ``A_t = diag(w_t) - (a_t u_t) u_t^T`` and adds ``k_t v_t^T``, so over a chunk with transition product
+    ``P = A_n ... A_1`` and own contribution ``S_loc`` (the chunk run from zeros), ``S_end = P S_begin + S_loc``.  Three
+    passes: (1) every chunk from zeros and, in further waves of the same launch, from the identity without the
+    ``k v^T`` term, all at once, no outputs, giving ``(S_loc, P)``; (2) the memory at every chunk's first token, chunk
+    after chunk, and the sequence's new carried memory; (3) every chunk again from its true memory, all at once,
+    writing outputs token by token."""
+    pcu_d, base_d, ident, zeros, ones, Pn = plan
+    H, dk, dv = r.shape[1], r.shape[2], v.shape[2]
+    f32 = dict(dtype=torch.float32, device=r.device)
+    loc, prod = torch.empty(Pn, H, dk, dv, **f32), torch.empty(Pn, H, dk, dk, **f32)
+    nat.delta_scan(r, k, v, zw, w0, za, ab, decay_coef, key_eps, loc, ident, pcu_d, zeros, prod, False, True)
+    init = torch.empty_like(loc)
+    nat.delta_chunk_combine(S, state_slots, start, base_d, loc, prod, init)
+    return nat.delta_scan(r, k, v, zw, w0, za, ab, decay_coef, key_eps, init, ident, pcu_d, ones, None, True, False)
 
 
 def tanh_act(x):
