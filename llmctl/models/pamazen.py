@@ -97,7 +97,7 @@ class PamazenConfig:
                 raise ValueError(f"unknown feed-forward kind {mlp.get('kind')!r}")
             m = spec["mixer"]
             if spec["type"] == "attention" and m.get("v_mix"):
-                widths.add(int(m.get("kv_heads", m["heads"])) * int(m["vdim"]))
+                widths.add((int(m.get("kv_heads", m["heads"])), int(m["vdim"])))
         if len(widths) > 1:
             raise ValueError("layers that mix their values with the first one's need values of one size")
         return cls(extra=d, **kw)
@@ -170,6 +170,9 @@ class PamazenLayer(nn.Module):
         self.norm1 = nn.Parameter(torch.ones(1, **f32))  # an RMS norm with one weight for all coordinates
         self.hc1 = HyperConnection(S, device)
         self.mixer = MIXER_TYPES[spec["type"]](W, spec["mixer"], cfg.layer_norm_eps, cfg.decay_ranks.get(i), role, **kw)
+        # a checkpoint carries a mixing factor for every attention layer; layers that do not mix keep theirs unread
+        self.vmix_unread = (nn.Parameter(torch.zeros(1, **f32))
+                            if spec["type"] == "attention" and self.mixer.vmix is None else None)
         mlp = spec.get("mlp")
         self.ff = None
         if mlp is not None:
@@ -318,8 +321,8 @@ class PamazenLM(nn.Module):
             else:
                 put(m.w_qkv, torch.cat([W[q + "q"], W[q + "k"], W[q + "v"]], 0))
                 put(m.w_o, W[q + "o"])
-                if m.vmix is not None:
-                    put(m.vmix, W[q + "vmix"])
+                if q + "vmix" in W:
+                    put(m.vmix if m.vmix is not None else layer.vmix_unread, W[q + "vmix"])
             ff, f = layer.ff, p + "mlp."
             if ff is None:
                 continue
@@ -362,7 +365,7 @@ class PamazenLM(nn.Module):
             else:
                 a, c = m.H * m.dk, (m.H + m.G) * m.dk
                 out.update({q + "q": m.w_qkv[:a], q + "k": m.w_qkv[a:c], q + "v": m.w_qkv[c:], q + "o": m.w_o})
-                out[q + "vmix"] = m.vmix.reshape(()) if m.vmix is not None else torch.zeros(())
+                out[q + "vmix"] = (m.vmix if m.vmix is not None else layer.vmix_unread).reshape(())
             ff, f = layer.ff, p + "mlp."
             if ff is None:
                 continue

@@ -23,12 +23,15 @@ def gelu_tanh(z):
 
 
 def rotate_pairs(x, base, dims, factor):
-    """x [T, H, d]: neighbours (2i, 2i + 1), i < dims / 2, are turned by p * base^(-2i / dims) / factor."""
-    T = x.shape[0]
+    """x [T, H, d]: neighbours (2i, 2i + 1), i < dims / 2, are turned by p * base^(-2i / dims) / factor, p = 0 .. T-1."""
+    return rotate_pairs_at(x, torch.arange(x.shape[0], dtype=F64), base, dims, factor)
+
+
+def rotate_pairs_at(x, pos, base, dims, factor):
     out = x.clone()
     for i in range(dims // 2):
         f = float(base) ** (-2.0 * i / dims) / factor
-        ang = torch.arange(T, dtype=F64) * f
+        ang = pos * f
         c, s = torch.cos(ang)[:, None], torch.sin(ang)[:, None]
         u, v = x[:, :, 2 * i], x[:, :, 2 * i + 1]
         out[:, :, 2 * i] = u * c - v * s
