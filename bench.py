@@ -69,13 +69,19 @@ def parse():
                     help="instead of the training benchmark: serving prefill / decode throughput of Malinex "
                          "configurations beside Lenitar at equal size (comma-separated sizes of "
                          "llmctl.benchmarks.hybrid.MALINEX_SIZES, or 'all'); one JSON line per size")
+    ap.add_argument("--pamazen-compare", default=None, metavar="SIZES",
+                    help="instead of the training benchmark: serving prefill / decode throughput of Pamazen "
+                         "configurations beside Malinex at equal size (comma-separated sizes of "
+                         "llmctl.benchmarks.hybrid.PAMAZEN_SIZES, or 'all'); one JSON line per size")
     return ap.parse_args()
 
 
 def hybrid_compare(args) -> None:
     from llmctl.benchmarks import hybrid
 
-    if args.malinex_compare:
+    if args.pamazen_compare:
+        table, which, family = hybrid.PAMAZEN_SIZES, args.pamazen_compare, "pamazen"
+    elif args.malinex_compare:
         table, which, family = hybrid.MALINEX_SIZES, args.malinex_compare, "malinex"
     elif args.dumalix_compare:
         table, which, family = hybrid.DUMALIX_SIZES, args.dumalix_compare, "dumalix"
@@ -88,7 +94,7 @@ def hybrid_compare(args) -> None:
 
 def main():
     args = parse()
-    if args.hybrid_compare or args.dumalix_compare or args.malinex_compare:
+    if args.hybrid_compare or args.dumalix_compare or args.malinex_compare or args.pamazen_compare:
         return hybrid_compare(args)
     import torch
     import torch.distributed as dist

@@ -3,7 +3,10 @@ transformer: softmax attention + top-k SwiGLU experts) at equal width, depth, he
 a Dumalix configuration beside the dense transformer (grouped-query softmax attention + SwiGLU) at equal
 width, layer runs, heads, kv heads and feed-forward size, and of a Malinex configuration beside Lenitar (the
 closest existing model: recurrent-state layers among attention layers, routed experts, an fp32 residual
-stream) at equal width, depth, heads, experts and expert size.
+stream) at equal width, depth, heads, experts and expert size, and of a Pamazen configuration beside Malinex (the
+closest existing model: grouped-query attention over paged rows beside a decayed matrix memory in state slots,
+softmax-routed experts with a shared one, an fp32 residual stream) at equal width, depth, heads, kv heads, experts
+and expert size.
 
 Both run through the same engine calls: one prompt portion per sequence (``InferenceEngine.prefill``)
 and then one-token decode steps of the whole batch (``InferenceEngine.decode``); random weights,
@@ -44,6 +47,30 @@ MALINEX_SIZES = {
     "small": dict(width=1024, layers=6, heads=8, kv_heads=2, head_dim=128, experts=8, top=2, ff=512, prompt=2048, batch=16),
     "medium": dict(width=2048, layers=6, heads=16, kv_heads=4, head_dim=128, experts=8, top=2, ff=1024, prompt=2048, batch=16),
 }  # (no width 4096: Lenitar's latent rank of width / 4 is then beyond its attention kernels)
+
+
+# Pamazen: width, layers (every third is the parallel pair of windowed attention and delta-rule memory, the others
+# rotary attention), heads of ``head_dim`` (delta rule: heads of half that), kv heads, routed gated experts + one shared,
+# four residual streams, window, prompt, decode batch
+PAMAZEN_SIZES = {
+    "tiny": dict(width=128, layers=3, heads=4, kv_heads=2, head_dim=32, experts=4, top=2, ff=64, window=32, prompt=64, batch=2),
+    "small": dict(width=1024, layers=6, heads=8, kv_heads=2, head_dim=128, experts=8, top=2, ff=512, window=1024, prompt=2048, batch=16),
+    "medium": dict(width=2048, layers=6, heads=16, kv_heads=4, head_dim=128, experts=8, top=2, ff=1024, window=1024, prompt=2048, batch=16),
+    "large": dict(width=4096, layers=6, heads=32, kv_heads=8, head_dim=128, experts=8, top=2, ff=2048, window=1024, prompt=4096, batch=16),
+}
+
+
+def _configs_pamazen(s: Dict):
+    from llmctl.models.malinex import malinex_template
+    from llmctl.models.pamazen import pamazen_template
+
+    pa = pamazen_template(width=s["width"], layers=s["layers"], heads=s["heads"], kv_heads=s["kv_heads"], vocab=32000, every=3,
+                          experts=s["experts"], top=s["top"], expert_ff=s["ff"], head_dim=s["head_dim"], streams=4, window=s["window"])
+    pa.max_position_embeddings = s["prompt"] + 256
+    ma = malinex_template(width=s["width"], layers=s["layers"], heads=s["heads"], kv_heads=s["kv_heads"], vocab=32000, every=3,
+                          experts=s["experts"], top=s["top"], expert_ff=s["ff"], head_dim=s["head_dim"],
+                          max_positions=s["prompt"] + 256)
+    return pa, ma
 
 
 def _configs_malinex(s: Dict):
@@ -151,7 +178,12 @@ def _measure(eng, prompt: int, batch: int, steps: int, warmup: int) -> Dict[str,
 def run(sizes: List[str], device: str = "auto", steps: int = 5, warmup: int = 2, family: str = "lenitar") -> List[Dict]:
     out = []
     for name in sizes:
-        if family == "malinex":
+        if family == "pamazen":
+            s = PAMAZEN_SIZES[name]
+            hy, tr = _configs_pamazen(s)
+            row = {"size": name, **s}
+            pair = (("pamazen", hy), ("malinex", tr))
+        elif family == "malinex":
             s = MALINEX_SIZES[name]
             hy, tr = _configs_malinex(s)
             row = {"size": name, **s}

@@ -332,10 +332,11 @@ def test_far_keys_window_edges_and_kept_tokens(dev, form, bs, L, j0, window, kee
     # the standing-out key lies far back, among the kept first tokens or just past them, just inside or just outside the
     # last queries' windows, on either side of page and 64-key-tile borders
     device, dtype, _ = dev
-    tol = 1e-4 if dtype == torch.float32 else 4e-2
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
     for mfma in ([True, False] if (device == "cuda" and dtype == torch.bfloat16) else [True]):
         got, want = _window_case(device, dtype, bs, L, j0, form, mfma, window, keep)
-        assert float((got - want).abs().max()) < tol, (mfma, float((got - want).abs().max()))
+        err = float((got - want).abs().max()) / max(1.0, float(want.abs().max()))  # (the standing-out value is ~9)
+        assert err < tol, (mfma, err)
 
 
 @pytest.mark.gpu
@@ -346,7 +347,7 @@ def test_capped_windowed_attention_kernels_gpu(H, G, dk):
         for form in ("prefill", "decode"):
             for mfma in (True, False):
                 got, want = _window_case("cuda", dtype, 16, 300, 2, form, mfma, 90, 4, H=H, G=G, dk=dk)
-                assert float((got - want).abs().max()) < tol, (dtype, form, mfma)
+                assert float((got - want).abs().max()) / max(1.0, float(want.abs().max())) < tol, (dtype, form, mfma)
 
 
 def _memory_case(device, dtype, T, dk, dv, H, cuts, far, chunked):
