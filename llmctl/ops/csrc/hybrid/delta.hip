@@ -10,7 +10,8 @@
 //                        without the k v^T term: that is the product of the tokens' transition matrices
 //                        A_t = diag(w_t) - (a_t u_t) u_t^T, which carries a memory across the sequence's tokens.
 //   delta_chunk_combine  the memory at the first token of every chunk of a portion from the chunks' own contributions
-//                        and transition products (S_end = P S_begin + S_loc), and the sequence's new carried memory.
+//                        and transition products (S_end = P S_begin + S_loc), and the sequence's new carried memory
+//                        (a small matrix product per chunk, register-tiled out of LDS).
 #include "hybrid_common.h"
 
 namespace llmctl_hybrid {
@@ -33,7 +34,7 @@ struct DeltaArgs {
   const int* slots;
   const int* cu;
   const int* start;
-  float* P;    // nullptr, or [sequences, H, dk, dk]: the product of the transition matrices of the sequence's tokens
+  float* P;    // nullptr, or [sequences, H, dk, dk]: the product of the transition matrices of the sequence's tokens, transposed
   float* out;  // nullptr, or [T, H, dv]
   int H, dk, dv, write_state;
 };
@@ -166,7 +167,7 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs a) {
       float* Pb = a.P + ((int64_t)sq * H + h) * dk * dk;
 #pragma unroll
       for (int d = 0; d < KT; ++d)
-        if (d < dk) Pb[(int64_t)d * dk + col] = S[d];
+        if (d < dk) Pb[(int64_t)col * dk + d] = S[d];  // transposed: the combine pass reads rows of P^T
     }
   } else if (a.write_state && cok) {
 #pragma unroll
@@ -175,40 +176,89 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs a) {
   }
 }
 
-// Sequence s has chunks [base[s], base[s+1]); chunk p run from zeros left loc[p] and its transition product P[p].
-// For every chunk the memory at its first token goes to init[p]: the sequence's carried memory (zeros at
-// position 0) for its first chunk, then S' = P S + loc; what follows the last chunk is the sequence's new carried
-// memory.  One workgroup per (sequence, head); the running memory lives in LDS (two copies), chunks in order.
-__global__ __launch_bounds__(256) void delta_chunk_combine_kernel(float* __restrict__ Sp, const int* __restrict__ slots,
-                                                                  const int* __restrict__ start, const int* __restrict__ base,
-                                                                  const float* __restrict__ loc, const float* __restrict__ P,
-                                                                  float* __restrict__ init, int H, int dk, int dv) {
-  extern __shared__ float cur[];  // [2][dk * dv]
-  const int s = blockIdx.x, h = blockIdx.y;
-  if (base[s] == base[s + 1]) return;
-  const int per = dk * dv;
+// Sequence s has chunks [base[s], base[s+1]); chunk p run from zeros left loc[p] and its transition product, stored
+// transposed: Pt[p][j][d] = P[d][j].  For every chunk the memory at its first token goes to init[p]: the sequence's
+// carried memory (zeros at position 0) for its first chunk, then S' = P S + loc; what follows the last chunk is the
+// sequence's new carried memory.  One workgroup per (sequence, head), chunks in order: the running memory [dk, dv] and
+// the chunk's Pt live in LDS, a thread owns 4 x 4 tiles of the product (both operands read as 16-byte rows), and the
+// next chunk's Pt is fetched into registers while this chunk's product runs.  dk and dv are multiples of 4.
+constexpr int CB_NT = 256;
+constexpr int CB_PRE = 48;   // Pt entries a thread fetches ahead: dk * dk <= CB_PRE * CB_NT
+constexpr int CB_TILES = 2;  // 4 x 4 tiles per thread: dk * dv <= 16 * CB_TILES * CB_NT
+
+__global__ __launch_bounds__(CB_NT) void delta_chunk_combine_kernel(float* __restrict__ Sp, const int* __restrict__ slots,
+                                                                    const int* __restrict__ start, const int* __restrict__ base,
+                                                                    const float* __restrict__ loc, const float* __restrict__ Pt,
+                                                                    float* __restrict__ init, int H, int dk, int dv) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float* val = lds;            // [dk][dv]
+  float* pt = lds + dk * dv;   // [dk][dk], pt[j][d]
+  const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int p_lo = base[s], p_hi = base[s + 1];
+  if (p_lo == p_hi) return;
+  const int per = dk * dv, pp = dk * dk;
   float* real = Sp + ((int64_t)slots[s] * H + h) * per;
   const bool fresh = start[s] == 0;
-  for (int e = threadIdx.x; e < per; e += 256) cur[e] = fresh ? 0.f : real[e];
+  for (int e = tid; e < per; e += CB_NT) val[e] = fresh ? 0.f : real[e];
+  const int tcols = dv / 4, ntiles = (dk / 4) * tcols;
+  float pre[CB_PRE];
+  auto fetch = [&](int p) {
+    const float* src = Pt + ((int64_t)p * H + h) * pp;
+#pragma unroll
+    for (int i = 0; i < CB_PRE; ++i) {
+      const int e = tid + i * CB_NT;
+      pre[i] = e < pp ? src[e] : 0.f;
+    }
+  };
+  fetch(p_lo);
   __syncthreads();
-  int b = 0;
-  for (int p = base[s]; p < base[s + 1]; ++p) {
-    const float* val = cur + b * per;
-    float* nxt = cur + (b ^ 1) * per;
-    const float* Pp = P + ((int64_t)p * H + h) * dk * dk;
-    const float* lp = loc + ((int64_t)p * H + h) * per;
+  for (int p = p_lo; p < p_hi; ++p) {
     float* ip = init + ((int64_t)p * H + h) * per;
-    for (int e = threadIdx.x; e < per; e += 256) {
-      const int d = e / dv, c = e - d * dv;
-      ip[e] = val[e];
-      float acc = lp[e];
-      for (int j = 0; j < dk; ++j) acc += Pp[d * dk + j] * val[j * dv + c];
-      nxt[e] = acc;
+    for (int e = tid; e < per; e += CB_NT) ip[e] = val[e];
+#pragma unroll
+    for (int i = 0; i < CB_PRE; ++i) {
+      const int e = tid + i * CB_NT;
+      if (e < pp) pt[e] = pre[i];
     }
     __syncthreads();
-    b ^= 1;
+    if (p + 1 < p_hi) fetch(p + 1);
+    const float* lp = loc + ((int64_t)p * H + h) * per;
+    float acc[CB_TILES][4][4];
+#pragma unroll
+    for (int k = 0; k < CB_TILES; ++k) {
+      const int t = tid + k * CB_NT;
+      if (t < ntiles) {
+        const int d0 = (t / tcols) * 4, c0 = (t % tcols) * 4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float4 l4 = *reinterpret_cast<const float4*>(lp + (d0 + r) * dv + c0);
+          acc[k][r][0] = l4.x, acc[k][r][1] = l4.y, acc[k][r][2] = l4.z, acc[k][r][3] = l4.w;
+        }
+        for (int j = 0; j < dk; ++j) {
+          const float4 a4 = *reinterpret_cast<const float4*>(pt + j * dk + d0);
+          const float4 b4 = *reinterpret_cast<const float4*>(val + j * dv + c0);
+          const float a[4] = {a4.x, a4.y, a4.z, a4.w}, b[4] = {b4.x, b4.y, b4.z, b4.w};
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc[k][r][c] += a[r] * b[c];
+        }
+      }
+    }
+    __syncthreads();  // every read of this chunk's memory is done
+#pragma unroll
+    for (int k = 0; k < CB_TILES; ++k) {
+      const int t = tid + k * CB_NT;
+      if (t < ntiles) {
+        const int d0 = (t / tcols) * 4, c0 = (t % tcols) * 4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          *reinterpret_cast<float4*>(val + (d0 + r) * dv + c0) = make_float4(acc[k][r][0], acc[k][r][1], acc[k][r][2], acc[k][r][3]);
+      }
+    }
+    __syncthreads();
   }
-  for (int e = threadIdx.x; e < per; e += 256) real[e] = cur[b * per + e];
+  for (int e = tid; e < per; e += CB_NT) real[e] = val[e];
 }
 
 static void head_view(const at::Tensor& t, const char* name, int64_t T, int64_t H, at::ScalarType dt) {
@@ -284,10 +334,11 @@ void delta_chunk_combine(at::Tensor S, const at::Tensor& slots, const at::Tensor
   HYB_CHECK(i32(slots) && i32(start) && i32(base) && start.numel() == slots.numel() && base.numel() == slots.numel() + 1, "slots [n], start [n], base [n + 1]: int32");
   const int64_t ns = slots.numel();
   if (ns == 0 || Pn == 0) return;
-  const size_t lds = (size_t)2 * dk * dv * sizeof(float);
-  HYB_CHECK(lds <= 64 * 1024 && H <= 65535, "memory too large for the combine pass");
+  const size_t lds = (size_t)dk * (dk + dv) * sizeof(float);
+  HYB_CHECK(lds <= 64 * 1024 && H <= 65535 && dk % 4 == 0 && dv % 4 == 0 && dk * dk <= CB_PRE * CB_NT && dk * dv <= 16 * CB_TILES * CB_NT,
+            "combine pass: dk and dv multiples of 4, 4 dk (dk + dv) <= 64 KB");
   c10::DeviceGuard guard(S.device());
-  delta_chunk_combine_kernel<<<dim3((unsigned)ns, (unsigned)H), 256, lds, cur_stream()>>>(
+  delta_chunk_combine_kernel<<<dim3((unsigned)ns, (unsigned)H), CB_NT, lds, cur_stream()>>>(
       S.data_ptr<float>(), slots.data_ptr<int>(), start.data_ptr<int>(), base.data_ptr<int>(), loc.data_ptr<float>(), P.data_ptr<float>(),
       init.data_ptr<float>(), (int)H, (int)dk, (int)dv);
 }

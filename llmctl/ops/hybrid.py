@@ -395,14 +395,18 @@ def delta_scan(r, k, v, zw, w0, za, ab, decay_coef: float, key_eps: float, S, st
         nat = native_hybrid()
         if plan is None and cu_host is not None:
             plan = gla_chunk_plan(cu_host, r.device)
-        if plan is not None and DELTA_CHUNKED and k.shape[2] * v.shape[2] <= DELTA_COMBINE_MAX:
+        if plan is not None and DELTA_CHUNKED and _delta_combine_fits(k.shape[2], v.shape[2]):
             return _delta_scan_chunked(nat, r, k, v, zw, w0, za, ab, decay_coef, key_eps, S, state_slots, start, plan)
         return nat.delta_scan(r, k, v, zw, w0, za, ab, decay_coef, key_eps, S, state_slots, cu, start, None, True, True)
     return ref.delta_scan(r, k, v, zw, w0, za, ab, decay_coef, key_eps, S, state_slots, cu, start)
 
 
 DELTA_CHUNKED = True  # long portions run chunk-parallel
-DELTA_COMBINE_MAX = 8192  # memory entries per head that the combine pass holds twice in LDS
+
+
+def _delta_combine_fits(dk: int, dv: int) -> bool:
+    """The combine pass holds a head's memory and a chunk's transition product in LDS and tiles them 4 x 4."""
+    return dk % 4 == 0 and dv % 4 == 0 and 4 * dk * (dk + dv) <= 65536 and dk * dk <= 48 * 256 and dk * dv <= 8192
 
 
 def _delta_scan_chunked(nat, r, k, v, zw, w0, za, ab, decay_coef, key_eps, S, state_slots, start, plan):
@@ -410,7 +414,7 @@ def _delta_scan_chunked(nat, r, k, v, zw, w0, za, ab, decay_coef, key_eps, S, st
     maps it by ``A_t = diag(w_t) - (a_t u_t) u_t^T`` and adds ``k_t v_t^T``, so over a chunk with transition product
     ``P = A_n ... A_1`` and own contribution ``S_loc`` (the chunk run from zeros), ``S_end = P S_begin + S_loc``.  Three
     passes: (1) every chunk from zeros and, in further waves of the same launch, from the identity without the
-    ``k v^T`` term, all at once, no outputs, giving ``(S_loc, P)``; (2) the memory at every chunk's first token, chunk
+    ``k v^T`` term, all at once, no outputs, giving ``(S_loc, P^T)``; (2) the memory at every chunk's first token, chunk
     after chunk, and the sequence's new carried memory; (3) every chunk again from its true memory, all at once,
     writing outputs token by token."""
     pcu_d, base_d, ident, zeros, ones, Pn = plan

@@ -398,14 +398,14 @@ def _memory_case(device, dtype, T, dk, dv, H, cuts, far, chunked):
 def test_memory_survives_and_forgets(dev, T, cuts, far):
     device, dtype, _ = dev
     tol = 2e-4 if dtype == torch.float32 else 3e-2
-    H, dk, dv = 3, 10, 12
+    H, dk, dv = 3, 12, 20
     for chunked in ([False, True] if device == "cuda" else [False]):
         got, want, S, S_end, keep = _memory_case(device, dtype, T, dk, dv, H, cuts, far, chunked)
         scale = float(want.abs().max())
         assert float((got - want).abs().max()) / scale < tol, chunked
         assert float((S - S_end).abs().max()) / float(S_end.abs().max()) < tol, chunked
         # the kept channel still holds token ``far``'s value after T tokens; the last outputs are made of it
-        assert float(want[T - 1].abs().max()) > 10.0 * float(want[T - 20].abs().max())
+        assert float(want[T - 1].abs().max()) > 5.0 * float(want[T - 20].abs().max())
 
 
 @pytest.mark.gpu
