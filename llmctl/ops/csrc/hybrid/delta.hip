@@ -210,7 +210,25 @@ __global__ __launch_bounds__(CB_NT) void delta_chunk_combine_kernel(float* __res
       pre[i] = e < pp ? src[e] : 0.f;
     }
   };
+  // the chunk's own contribution, fetched a chunk ahead like its Pt: the accumulators start from it
+  float nl[CB_TILES][4][4];
+  auto fetch_loc = [&](int p) {
+    const float* lp = loc + ((int64_t)p * H + h) * per;
+#pragma unroll
+    for (int k = 0; k < CB_TILES; ++k) {
+      const int t = tid + k * CB_NT;
+      if (t < ntiles) {
+        const int d0 = (t / tcols) * 4, c0 = (t % tcols) * 4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float4 l4 = *reinterpret_cast<const float4*>(lp + (d0 + r) * dv + c0);
+          nl[k][r][0] = l4.x, nl[k][r][1] = l4.y, nl[k][r][2] = l4.z, nl[k][r][3] = l4.w;
+        }
+      }
+    }
+  };
   fetch(p_lo);
+  fetch_loc(p_lo);
   __syncthreads();
   for (int p = p_lo; p < p_hi; ++p) {
     float* ip = init + ((int64_t)p * H + h) * per;
@@ -221,19 +239,23 @@ __global__ __launch_bounds__(CB_NT) void delta_chunk_combine_kernel(float* __res
       if (e < pp) pt[e] = pre[i];
     }
     __syncthreads();
-    if (p + 1 < p_hi) fetch(p + 1);
-    const float* lp = loc + ((int64_t)p * H + h) * per;
     float acc[CB_TILES][4][4];
+#pragma unroll
+    for (int k = 0; k < CB_TILES; ++k)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[k][r][c] = nl[k][r][c];
+    if (p + 1 < p_hi) {
+      fetch(p + 1);
+      fetch_loc(p + 1);
+    }
 #pragma unroll
     for (int k = 0; k < CB_TILES; ++k) {
       const int t = tid + k * CB_NT;
       if (t < ntiles) {
         const int d0 = (t / tcols) * 4, c0 = (t % tcols) * 4;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float4 l4 = *reinterpret_cast<const float4*>(lp + (d0 + r) * dv + c0);
-          acc[k][r][0] = l4.x, acc[k][r][1] = l4.y, acc[k][r][2] = l4.z, acc[k][r][3] = l4.w;
-        }
+#pragma unroll 4
         for (int j = 0; j < dk; ++j) {
           const float4 a4 = *reinterpret_cast<const float4*>(pt + j * dk + d0);
           const float4 b4 = *reinterpret_cast<const float4*>(val + j * dv + c0);
