@@ -187,28 +187,41 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs a) {
 // Sequence s has chunks [base[s], base[s+1]); chunk p run from zeros left loc[p] and its transition product, stored
 // transposed: Pt[p][j][d] = P[d][j].  For every chunk the memory at its first token goes to init[p]: the sequence's
 // carried memory (zeros at position 0) for its first chunk, then S' = P S + loc; what follows the last chunk is the
-// sequence's new carried memory.  One workgroup per (sequence, head), chunks in order: the running memory [dk, dv] and
-// the chunk's Pt live in LDS, a thread owns 4 x 4 tiles of the product (both operands read as 16-byte rows), and the
-// next chunk's Pt is fetched into registers while this chunk's product runs.  dk and dv are multiples of 4.
+// sequence's new carried memory.  The columns of a memory are independent under P, so a workgroup owns (sequence,
+// head, ``cpb`` value columns) and walks the chunks in order: its columns of the running memory [dk, cpb] and the
+// chunk's Pt live in LDS, a thread owns a 4 x 4 tile of the product (both operands read as 16-byte rows) over a
+// ``JG``-th of the sum, the parts are added through LDS, and the next chunk's Pt and loc are fetched into registers
+// while this chunk's product runs.  dk, dv and cpb are multiples of 4.
 constexpr int CB_NT = 256;
 constexpr int CB_PRE = 48;   // Pt entries a thread fetches ahead: dk * dk <= CB_PRE * CB_NT
-constexpr int CB_TILES = 2;  // 4 x 4 tiles per thread: dk * dv <= 16 * CB_TILES * CB_NT
+constexpr int CB_TILES = 2;  // 4 x 4 tiles per thread when one thread sums all of j: dk * cpb <= 16 * CB_TILES * CB_NT
 
 __global__ __launch_bounds__(CB_NT) void delta_chunk_combine_kernel(float* __restrict__ Sp, const int* __restrict__ slots,
                                                                     const int* __restrict__ start, const int* __restrict__ base,
                                                                     const float* __restrict__ loc, const float* __restrict__ Pt,
-                                                                    float* __restrict__ init, int H, int dk, int dv) {
+                                                                    float* __restrict__ init, int H, int dk, int dv, int cpb, int JG) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  float* val = lds;            // [dk][dv]
-  float* pt = lds + dk * dv;   // [dk][dk], pt[j][d]
-  const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int s = blockIdx.x, h = blockIdx.y, cb = blockIdx.z * cpb, tid = threadIdx.x;
   const int p_lo = base[s], p_hi = base[s + 1];
   if (p_lo == p_hi) return;
-  const int per = dk * dv, pp = dk * dk;
+  const int per = dk * dv, pp = dk * dk, mine = dk * cpb;
+  const int tcols = cpb / 4, ntiles = (dk / 4) * tcols;
+  float* val = lds;             // [dk][cpb]
+  float* pt = lds + mine;       // [dk][dk], pt[j][d]
+  float* red = pt + pp;         // [JG - 1][ntiles][16]
+  // this thread's tiles and its part of the sum
+  const int g = JG > 1 ? tid / ntiles : 0;
+  int tile[CB_TILES];
+#pragma unroll
+  for (int k = 0; k < CB_TILES; ++k) {
+    if (JG > 1) tile[k] = (k == 0 && g < JG) ? tid % ntiles : -1;
+    else tile[k] = tid + k * CB_NT < ntiles ? tid + k * CB_NT : -1;
+  }
+  const int jlen = (dk + JG - 1) / JG;
+  const int j_lo = min(g * jlen, dk), j_hi = min(j_lo + jlen, dk);
   float* real = Sp + ((int64_t)slots[s] * H + h) * per;
   const bool fresh = start[s] == 0;
-  for (int e = tid; e < per; e += CB_NT) val[e] = fresh ? 0.f : real[e];
-  const int tcols = dv / 4, ntiles = (dk / 4) * tcols;
+  for (int e = tid; e < mine; e += CB_NT) val[e] = fresh ? 0.f : real[(e / cpb) * dv + cb + e % cpb];
   float pre[CB_PRE];
   auto fetch = [&](int p) {
     const float* src = Pt + ((int64_t)p * H + h) * pp;
@@ -218,15 +231,14 @@ __global__ __launch_bounds__(CB_NT) void delta_chunk_combine_kernel(float* __res
       pre[i] = e < pp ? src[e] : 0.f;
     }
   };
-  // the chunk's own contribution, fetched a chunk ahead like its Pt: the accumulators start from it
+  // the chunk's own contribution, fetched a chunk ahead like its Pt (by the threads that finish the sums)
   float nl[CB_TILES][4][4];
   auto fetch_loc = [&](int p) {
-    const float* lp = loc + ((int64_t)p * H + h) * per;
+    const float* lp = loc + ((int64_t)p * H + h) * per + cb;
 #pragma unroll
     for (int k = 0; k < CB_TILES; ++k) {
-      const int t = tid + k * CB_NT;
-      if (t < ntiles) {
-        const int d0 = (t / tcols) * 4, c0 = (t % tcols) * 4;
+      if (tile[k] >= 0 && g == 0) {
+        const int d0 = (tile[k] / tcols) * 4, c0 = (tile[k] % tcols) * 4;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const float4 l4 = *reinterpret_cast<const float4*>(lp + (d0 + r) * dv + c0);
@@ -235,18 +247,23 @@ __global__ __launch_bounds__(CB_NT) void delta_chunk_combine_kernel(float* __res
       }
     }
   };
+#pragma unroll
+  for (int k = 0; k < CB_TILES; ++k)
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) nl[k][r][c] = 0.f;
   fetch(p_lo);
   fetch_loc(p_lo);
-  __syncthreads();
   for (int p = p_lo; p < p_hi; ++p) {
-    float* ip = init + ((int64_t)p * H + h) * per;
-    for (int e = tid; e < per; e += CB_NT) ip[e] = val[e];
 #pragma unroll
     for (int i = 0; i < CB_PRE; ++i) {
       const int e = tid + i * CB_NT;
       if (e < pp) pt[e] = pre[i];
     }
-    __syncthreads();
+    __syncthreads();  // this chunk's Pt and the memory before it are in LDS
+    float* ip = init + ((int64_t)p * H + h) * per + cb;
+    for (int e = tid; e < mine; e += CB_NT) ip[(e / cpb) * dv + e % cpb] = val[e];
     float acc[CB_TILES][4][4];
 #pragma unroll
     for (int k = 0; k < CB_TILES; ++k)
@@ -260,13 +277,12 @@ __global__ __launch_bounds__(CB_NT) void delta_chunk_combine_kernel(float* __res
     }
 #pragma unroll
     for (int k = 0; k < CB_TILES; ++k) {
-      const int t = tid + k * CB_NT;
-      if (t < ntiles) {
-        const int d0 = (t / tcols) * 4, c0 = (t % tcols) * 4;
+      if (tile[k] >= 0) {
+        const int d0 = (tile[k] / tcols) * 4, c0 = (tile[k] % tcols) * 4;
 #pragma unroll 4
-        for (int j = 0; j < dk; ++j) {
+        for (int j = j_lo; j < j_hi; ++j) {
           const float4 a4 = *reinterpret_cast<const float4*>(pt + j * dk + d0);
-          const float4 b4 = *reinterpret_cast<const float4*>(val + j * dv + c0);
+          const float4 b4 = *reinterpret_cast<const float4*>(val + j * cpb + c0);
           const float a[4] = {a4.x, a4.y, a4.z, a4.w}, b[4] = {b4.x, b4.y, b4.z, b4.w};
 #pragma unroll
           for (int r = 0; r < 4; ++r)
@@ -275,20 +291,35 @@ __global__ __launch_bounds__(CB_NT) void delta_chunk_combine_kernel(float* __res
         }
       }
     }
-    __syncthreads();  // every read of this chunk's memory is done
+    if (JG > 1 && g > 0 && tile[0] >= 0) {
+      float* rp = red + ((g - 1) * ntiles + tile[0]) * 16;
 #pragma unroll
-    for (int k = 0; k < CB_TILES; ++k) {
-      const int t = tid + k * CB_NT;
-      if (t < ntiles) {
-        const int d0 = (t / tcols) * 4, c0 = (t % tcols) * 4;
+      for (int r = 0; r < 4; ++r) *reinterpret_cast<float4*>(rp + 4 * r) = make_float4(acc[0][r][0], acc[0][r][1], acc[0][r][2], acc[0][r][3]);
+    }
+    __syncthreads();  // every read of this chunk's memory and Pt is done; the parts of the sums are in LDS
+    if (g == 0) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          *reinterpret_cast<float4*>(val + (d0 + r) * dv + c0) = make_float4(acc[k][r][0], acc[k][r][1], acc[k][r][2], acc[k][r][3]);
+      for (int k = 0; k < CB_TILES; ++k) {
+        if (tile[k] >= 0) {
+          const int d0 = (tile[k] / tcols) * 4, c0 = (tile[k] % tcols) * 4;
+          if (k == 0)
+            for (int gg = 1; gg < JG; ++gg) {
+              const float* rp = red + ((gg - 1) * ntiles + tile[0]) * 16;
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const float4 x4 = *reinterpret_cast<const float4*>(rp + 4 * r);
+                acc[0][r][0] += x4.x, acc[0][r][1] += x4.y, acc[0][r][2] += x4.z, acc[0][r][3] += x4.w;
+              }
+            }
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            *reinterpret_cast<float4*>(val + (d0 + r) * cpb + c0) = make_float4(acc[k][r][0], acc[k][r][1], acc[k][r][2], acc[k][r][3]);
+        }
       }
     }
-    __syncthreads();
   }
-  for (int e = tid; e < per; e += CB_NT) real[e] = val[e];
+  __syncthreads();
+  for (int e = tid; e < mine; e += CB_NT) real[(e / cpb) * dv + cb + e % cpb] = val[e];
 }
 
 static void head_view(const at::Tensor& t, const char* name, int64_t T, int64_t H, at::ScalarType dt) {
@@ -364,13 +395,18 @@ void delta_chunk_combine(at::Tensor S, const at::Tensor& slots, const at::Tensor
   HYB_CHECK(i32(slots) && i32(start) && i32(base) && start.numel() == slots.numel() && base.numel() == slots.numel() + 1, "slots [n], start [n], base [n + 1]: int32");
   const int64_t ns = slots.numel();
   if (ns == 0 || Pn == 0) return;
-  const size_t lds = (size_t)dk * (dk + dv) * sizeof(float);
-  HYB_CHECK(lds <= 64 * 1024 && H <= 65535 && dk % 4 == 0 && dv % 4 == 0 && dk * dk <= CB_PRE * CB_NT && dk * dv <= 16 * CB_TILES * CB_NT,
-            "combine pass: dk and dv multiples of 4, 4 dk (dk + dv) <= 64 KB");
+  HYB_CHECK(dk % 4 == 0 && dv % 4 == 0 && dk * dk <= CB_PRE * CB_NT, "combine pass: dk and dv multiples of 4, dk * dk <= 12288");
+  // value columns per workgroup; parts of the sum per tile when a workgroup has fewer tiles than threads
+  const int64_t cpb = (dv % 16 == 0 && dv > 16) ? 16 : dv;
+  const int64_t ntiles = (dk / 4) * (cpb / 4);
+  const int64_t JG = ntiles >= CB_NT ? 1 : std::min<int64_t>(4, CB_NT / ntiles);
+  HYB_CHECK(ntiles <= CB_TILES * CB_NT, "combine pass: dk * dv too large");
+  const size_t lds = (size_t)(dk * cpb + dk * dk + (JG - 1) * ntiles * 16) * sizeof(float);
+  HYB_CHECK(lds <= 64 * 1024 && H <= 65535, "memory too large for the combine pass");
   c10::DeviceGuard guard(S.device());
-  delta_chunk_combine_kernel<<<dim3((unsigned)ns, (unsigned)H), CB_NT, lds, cur_stream()>>>(
+  delta_chunk_combine_kernel<<<dim3((unsigned)ns, (unsigned)H, (unsigned)(dv / cpb)), CB_NT, lds, cur_stream()>>>(
       S.data_ptr<float>(), slots.data_ptr<int>(), start.data_ptr<int>(), base.data_ptr<int>(), loc.data_ptr<float>(), P.data_ptr<float>(),
-      init.data_ptr<float>(), (int)H, (int)dk, (int)dv);
+      init.data_ptr<float>(), (int)H, (int)dk, (int)dv, (int)cpb, (int)JG);
 }
 
 }  // namespace llmctl_hybrid
