@@ -103,20 +103,12 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs a) {
       for (int i = 0; i < NR; ++i) {
         kc[j][i] = kn[j][i];
         rc[j][i] = rn[j][i];
-        wc[j][i] = 1.f;
-        ac[j][i] = 0.f;
+        wc[j][i] = expf(-a.coef * sigm(zn[j][i] + w0[i]));
+        ac[j][i] = sigm(an[j][i] + ab[i]);
         ss += kc[j][i] * kc[j][i];
       }
       vc[j] = vn[j];
-      inv[j] = 0.f;
-      if (t0 + j < t_b) {  // (a decode row is one token: the other seven cost nothing)
-#pragma unroll
-        for (int i = 0; i < NR; ++i) {
-          wc[j][i] = expf(-a.coef * sigm(zn[j][i] + w0[i]));
-          ac[j][i] = sigm(an[j][i] + ab[i]);
-        }
-        inv[j] = 1.0f / sqrtf(wave_sum(ss) + a.keps);  // up to eight independent reductions: off the token loop's path
-      }
+      inv[j] = 1.0f / sqrtf(wave_sum(ss) + a.keps);  // eight independent reductions: off the token loop's path
     }
     if (t0 + TB < t_b) fetch(t0 + TB);
 #pragma unroll

@@ -274,6 +274,16 @@ def test_long_portions(tmp_path, dev):
     check(tmp_path, dev, cfg, r, [[("a", 650), ("b", 10)], [("a", 49), ("b", 290)], [("a", 1)]], blocks=260)
 
 
+def test_heads_that_fit_the_matrix_cores(tmp_path, dev):
+    # head sizes in multiples of 8 (the bf16 runs take the matrix-core attention form), a prompt over several 64-key
+    # tiles, a window of 70 keys with 3 kept ones, then decoding, beside a short request
+    cfg = U.config([(U.att(heads=4, kv_heads=2, dim=32, vdim=16, rot_dims=16), None),
+                    (U.par(heads=4, kv_heads=1, dim=24, window=70, keep=3, rheads=2, rdim=16), None),
+                    (U.att(heads=4, kv_heads=2, dim=32, vdim=16, rot_dims=32, factor=None), None)], width=64, streams=4)
+    r = {"a": tokens(230, 50, 41), "b": tokens(9, 50, 42)}
+    check(tmp_path, dev, cfg, r, [[("a", 200), ("b", 4)]] + [[("a", 1), ("b", 1)]] * 5 + [[("a", 25)]], blocks=80)
+
+
 # ------------------------------------------------------------------ far keys and edges, at op level
 def _window_case(device, dtype, bs, L, j0, form, mfma, window, keep, cap=4.0, H=4, G=2, dk=16):
     """One key (position j0) stands out for the last queries; they see it if it lies in their window or among the kept

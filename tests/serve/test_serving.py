@@ -696,6 +696,7 @@ def test_sampling_oracle_property():
         if seed % 3 == 0:
             logits = logits.round()  # ties
         T, K, P = torch.tensor([temp]), torch.tensor([k]), torch.tensor([p])
+        p = float(P[0])  # the op sees the fp32 rounding (a p just below 1 becomes 1: no nucleus cut)
         lo, hi = min(u1, u2), max(u1, u2)
         a = int(ref.sample(logits, T, K, P, torch.tensor([lo]))[0])
         b = int(ref.sample(logits, T, K, P, torch.tensor([hi]))[0])
