@@ -9,8 +9,9 @@
 * :class:`GroupedAttention` — grouped-query softmax attention over a paged row cache ``[v | k]`` per
   kv head, with the options of small recent designs as parameters: short causal convolutions on the
   projected q / k / v, per-head RMS norm of q and k, rotary positions (neighbour or half pairs, YaRN
-  frequency scaling), values turned by their position and the head outputs turned back, a learned
-  per-head temperature, chunked or windowed masks, a softmax sink.
+  or linear frequency scaling), values turned by their position and the head outputs turned back, a learned
+  per-head temperature, capped scores, chunked or windowed masks, a window that spares the first tokens, a learned or
+  fixed softmax sink, values that are the key projection's output, values blended with an earlier layer's.
 * :class:`CausalConv` — a short causal convolution over time per channel, its last inputs carried in a
   state slot; :class:`ClampedGLU` — a gated feed-forward with clamped branches.
 * :class:`GatedLinearAttention` — a matrix memory per head whose key rows decay by a data-dependent
@@ -21,6 +22,11 @@
   grows with the logarithm of the position, a logarithmic distance penalty per head, key weights
   ``sigmoid(score + head bias)`` that are not normalised, one sigmoid output gate per head.
 * :class:`DenseFF` — an ungated feed-forward ``W_down act(W_up h)``.
+* :class:`DeltaRule` — the generalized delta rule: a matrix memory per head that decays per key channel, removes
+  what it holds along the current unit key at a learned rate and then writes ``k v^T``; low-rank decay projection
+  through a ``tanh``, per-head unit RMS, weight and sigmoid gate on the read-out; state in a slot pool.
+* :class:`ParallelMixers` — two mixers on the same input whose results are added with fixed factors (one input GEMM
+  on the stacked weights; paged rows for the one, state pools for the other).
 * :class:`MLSTM` — the xLSTM matrix memory: per head a ``[dk, dv]`` state with exponential input gate,
   sigmoid forget gate (both soft-capped) and a running log-scale stabiliser; state lives in a slot
   pool of the engine's cache, one slot per live sequence.

@@ -1,8 +1,8 @@
 """Ops of the hybrid sequence mixers: latent attention (compressed K/V cache, sliding window,
 softmax sink), grouped attention over paged rows (softmax or sigmoid weights, distance penalty), the
-mLSTM matrix memory, gated linear attention, the group-limited sigmoid router and the softmax router
-with a selection bias, and the fp32 residual stream of parallel layers and of layers with a gated
-residual between two norms.
+mLSTM matrix memory, gated linear attention, the generalized delta rule, the group-limited sigmoid router and the
+softmax router with a selection bias (optionally group-limited), and the fp32 residual stream of parallel layers, of
+layers with a gated residual between two norms, and of layers over several residual streams (hyper-connections).
 
 GPU tensors run the HIP kernels of ``csrc/hybrid`` (``torch.ops.llmctl_hybrid.*``, library
 ``_llmctl_hybrid.so``); CPU tensors run :mod:`llmctl.ops.ref_hybrid`.  All activations are
